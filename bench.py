@@ -1,0 +1,235 @@
+#!/usr/bin/env python3
+"""Benchmark of the W4A16 GEMM path on one MI355X.
+
+A "step" is one pass over the Llama-2-7B decode layer set: the four layer GEMMs
+(qkv, o, gate_up + SiLU, down + residual) at each of T = 1, 4, 8, 16 tokens = 16 launches,
+on a layer copy that differs from step to step (24 copies, about 2.5 GB of packed weights,
+so neither the L2s nor the 256 MB Infinity Cache can serve the weights).  The headline value
+is the aggregate achieved bandwidth: algorithmic bytes of all launches / elapsed time.
+
+Also reported in the same JSON line: the roofline of the dominant decode kernel (gate_up),
+the prefill (T = 2048) TFLOP/s of the same four shapes with the roofline of its dominant
+kernel, and the CPU baseline (the oracle: unpack, dequantise, torch fp32 matmul) timed on the
+host cores on a bounded sample.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16 matrix
+
+# name, K, N (gate_up: both halves), epilogue
+LAYER_7B = [("qkv", 4096, 12288, 0), ("o", 4096, 4096, 0), ("gate_up", 4096, 22016, 1), ("down", 11008, 4096, 2)]
+DECODE_T = (1, 4, 8, 16)
+PREFILL_T = 2048
+GROUP = 128
+
+
+def algorithmic_bytes(T, K, N, epi):
+    """int4 weights + fp16 scales + int4 zeros + activations + output (+ residual)."""
+    G = K // GROUP
+    n_out = N // 2 if epi == 1 else N
+    b = K * N // 2 + G * N * 2 + G * N // 2 + T * K * 2 + T * n_out * 2
+    if epi == 2:
+        b += T * N * 2
+    return b
+
+
+def flops(T, K, N):
+    return 2 * T * K * N
+
+
+def make_weights(tm, torch, gen, name, K, N):
+    """One copy of a layer matrix in the library's layout, from synthetic AWQ tensors on the GPU."""
+    G = K // GROUP
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=gen)
+    qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (G, N // 8), dtype=torch.int32, device="cuda", generator=gen)
+    s = (torch.randn((G, N), device="cuda", generator=gen).abs() * 0.01 + 1e-3).half()
+    if name == "gate_up":  # w1 and w3 (each [K, N/2]) interleaved by the repack path, as deploy does
+        fused = torch.empty_like(qw)
+        tm.fuse_w1_w3_s4_k_m8(qw.view(2 * K, N // 16), fused, N // 2, K)
+        qw = fused
+    A = torch.empty_like(qw)
+    Q = torch.empty((G, N), dtype=torch.int32, device="cuda")
+    tm.convert_s4_k_m8(A, Q, s, qw, s, qz, N, K, GROUP)
+    return A, Q
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=96)
+    ap.add_argument("--warmup", type=int, default=24)
+    ap.add_argument("--copies", type=int, default=24, help="distinct layer copies the steps rotate through")
+    ap.add_argument("--cold-gib", type=float, default=1.25,
+                    help="per-shape measurements rotate through at least this many GiB of weight copies")
+    ap.add_argument("--eager", action="store_true", help="launch from the host instead of replaying HIP graphs")
+    ap.add_argument("--prefill-steps", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-per-shape", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    import lmdeploy_amd.turbomind as tm
+
+    torch.cuda.set_device(0)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(20240611)
+    gemm = tm.GemmS4F16()
+    stream = torch.cuda.Stream()          # default priority; graphs are captured and replayed on it
+    shape = {name: (K, N, epi) for name, K, N, epi in LAYER_7B}
+    weights = {}
+    for name, K, N, epi in LAYER_7B:
+        per_copy = K * N // 2 + (K // GROUP) * N * 4
+        n = max(args.copies, int(args.cold_gib * 2 ** 30 / per_copy) + 1)
+        weights[name] = [make_weights(tm, torch, gen, name, K, N) for _ in range(n)]
+    Tmax = max(max(DECODE_T), PREFILL_T)
+    X = {K: torch.randn((Tmax, K), device="cuda", generator=gen).half() for K in (4096, 11008)}
+    Res = torch.randn((Tmax, 4096), device="cuda", generator=gen).half()
+    out = {name: torch.empty((Tmax, N // 2 if epi == 1 else N), dtype=torch.float16, device="cuda")
+           for name, K, N, epi in LAYER_7B}
+    torch.cuda.synchronize()
+
+    def launch(name, copy, T, st):
+        K, N, epi = shape[name]
+        A, Q = weights[name][copy % len(weights[name])]
+        gemm.Run(out[name], A, X[K], Q, N, T, K, GROUP, epi, -1, residual=Res if epi == 2 else None, stream=st)
+
+    def make_runner(work):
+        """work: list of launch lists; returns one callable per entry (a replayable HIP graph)."""
+        if args.eager:
+            return [lambda w=w: [launch(n, c, T, stream.cuda_stream) for n, c, T in w] for w in work]
+        runners = []
+        for w in work:
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                st = torch.cuda.current_stream().cuda_stream
+                for n, c, T in w:
+                    launch(n, c, T, st)
+            runners.append(g.replay)
+        return runners
+
+    def timed(runner, steps, warmup):
+        with torch.cuda.stream(stream):
+            for i in range(warmup):
+                runner[i % len(runner)]()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record(stream)
+            for i in range(steps):
+                runner[(warmup + i) % len(runner)]()
+            e1.record(stream)
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1)   # ms
+
+    # ---- headline: the decode layer set, one layer copy per step ------------------------------
+    step_bytes = sum(algorithmic_bytes(T, K, N, epi) for T in DECODE_T for _, K, N, epi in LAYER_7B)
+    runner = make_runner([[(name, c, T) for T in DECODE_T for name, _, _, _ in LAYER_7B] for c in range(args.copies)])
+    ms = timed(runner, args.steps, args.warmup)
+    ms_per_step = ms / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    def per_launch_us(name, tokens, passes=3):
+        """Average time of one launch of `name`, rotating through all of its copies (cold weights)."""
+        n = len(weights[name])
+        r = make_runner([[(name, c, tokens[c % len(tokens)]) for c in range(n)]])
+        return timed(r, passes, 1) * 1e3 / (passes * n)
+
+    # ---- roofline of the dominant decode kernel: gate_up alone, over >= cold-gib of copies -----
+    K, N, _ = shape["gate_up"]
+    gu_bytes = sum(algorithmic_bytes(T, K, N, 1) for T in DECODE_T) / len(DECODE_T)
+    gu_us = per_launch_us("gate_up", DECODE_T, passes=6)
+    achieved = gu_bytes / (gu_us * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "kernel": "decode_kernel, gate_up K=4096 N=22016 +SiLU, T cycling over {1,4,8,16}",
+                "bytes_per_launch": int(gu_bytes), "us_per_launch": round(gu_us, 3)}
+
+    # ---- per-shape decode table ----------------------------------------------------------------
+    per_shape = []
+    if not args.no_per_shape:
+        for name, K, N, epi in LAYER_7B:
+            for T in DECODE_T:
+                us = per_launch_us(name, (T,))
+                by = algorithmic_bytes(T, K, N, epi)
+                per_shape.append({"shape": name, "T": T, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
+                                  "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 3)})
+
+    # ---- prefill: T = 2048 ---------------------------------------------------------------------
+    prefill = None
+    if not args.no_prefill:
+        rows, tot_fl, tot_ms = [], 0.0, 0.0
+        for name, K, N, epi in LAYER_7B:
+            r = make_runner([[(name, c, PREFILL_T)] for c in range(4)])
+            t_ms = timed(r, args.prefill_steps, 3) / args.prefill_steps
+            fl = flops(PREFILL_T, K, N)
+            rows.append({"shape": name, "ms": round(t_ms, 4), "TFLOPs": round(fl / t_ms / 1e9, 1),
+                         "frac": round(fl / t_ms / 1e9 / MFMA_PEAK_TFLOPS, 4)})
+            tot_fl += fl
+            tot_ms += t_ms
+        dom = max(rows, key=lambda x: x["ms"])
+        prefill = {"T": PREFILL_T, "TFLOPs": round(tot_fl / tot_ms / 1e9, 1), "ms_per_layer": round(tot_ms, 4),
+                   "per_shape": rows,
+                   "roofline": {"bound": "mfma", "achieved": dom["TFLOPs"], "peak": MFMA_PEAK_TFLOPS,
+                                "unit": "TFLOP/s", "frac": dom["frac"], "traffic": None,
+                                "kernel": "prefill_kernel, %s, T=2048" % dom["shape"]}}
+
+    # ---- CPU baseline: the oracle on the host cores, one layer at T = 8 -------------------------
+    cpu = None
+    if not args.no_cpu:
+        import numpy as np
+        from oracle import w4a16_oracle as O
+        T = 8
+        t_deq = t_mm = 0.0
+        by = 0
+        for i, (name, K, N, epi) in enumerate(LAYER_7B):
+            d = O.make_inputs(77 + i, T, K, N, GROUP, residual=(epi == 2))
+            t0 = time.perf_counter()
+            W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], GROUP)
+            t1 = time.perf_counter()
+            O.epilogue(O.gemm_acc(d["X"], W), epi, d.get("R"))
+            t2 = time.perf_counter()
+            t_deq += t1 - t0
+            t_mm += t2 - t1
+            by += algorithmic_bytes(T, K, N, epi)
+        cpu = {"value": round(by / (t_deq + t_mm) / 1e9, 4), "unit": "GB/s", "cores": torch.get_num_threads(),
+               "kind": "port", "host_cpus": os.cpu_count(),
+               "sample": "one Llama-2-7B layer (qkv, o, gate_up+SiLU, down+residual) at T=8, single pass: "
+                         "numpy unpack+dequantise %.2f s (1 thread) + torch fp32 matmul+epilogue %.3f s (%d threads)"
+                         % (t_deq, t_mm, torch.get_num_threads())}
+
+    line = {
+        "metric": "W4A16 GEMM achieved HBM GB/s (M=1..16) + TFLOP/s (M=2048), % of roofline",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "Llama-2-7B decode layer set (qkv 4096x12288, o 4096x4096, gate_up 4096x22016 +SiLU, "
+                               "down 11008x4096 +residual) at T in {1,4,8,16}, group 128: 16 GEMMs per step, "
+                               "%d rotating layer copies" % args.copies,
+                   "launch": "eager" if args.eager else "hipgraph replay of one step",
+                   "bytes_per_step": step_bytes},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "roofline": roofline, "cpu_baseline": cpu, "decode_per_shape": per_shape, "prefill": prefill,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,139 @@
+/*
+ * C ABI of the MI355X (gfx950) W4A16 GEMM library, libw4a16.so.
+ *
+ * It replaces, for AMD CDNA4, TurboMind's `turbomind::GemmS4F16` operator and the
+ * `convert_s4` family of weight-repack functions of lmdeploy.  Every entry point takes
+ * plain pointers and sizes; device pointers are caller-owned HIP device memory and
+ * `stream` is a `hipStream_t` passed as `void*` (NULL = the default stream).  No entry
+ * point synchronises the device except `w4a16_measure`.  Functions return 0 on success
+ * or a negative W4A16_E* code and never throw; `w4a16_last_error()` returns a
+ * thread-local message for the last failure.
+ *
+ * Naming of sizes: `n_out` = output features (the reference's `m`), `tokens` = rows of
+ * the activation matrix (the reference's `n`), `k` = input features.  The reference
+ * passes them in that order: LlamaLinear.h:65-75 calls
+ * Run(out, kernel, in, scales_and_zeros, output_dims, batch_size, input_dims, ...).
+ */
+#ifndef W4A16_H_
+#define W4A16_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define W4A16_OK 0
+#define W4A16_EGROUP (-1)    /* unsupported group size (only 128)            */
+#define W4A16_ESHAPE (-2)    /* no feasible kernel for this shape            */
+#define W4A16_EHIP (-3)      /* the HIP runtime reported an error            */
+#define W4A16_EARG (-4)      /* null pointer / negative size / bad enum      */
+#define W4A16_EALGO (-5)     /* algo_id out of range                         */
+
+/* epilogues; 0 and 1 are GemmS4F16::Type (gemm_s4_f16.h:23-27), 2 is an extension */
+#define W4A16_GEMM 0
+#define W4A16_FUSED_SILU_FFN 1
+#define W4A16_FUSED_ADD 2
+
+typedef struct w4a16_handle w4a16_handle;
+
+/* One row of `w4a16_measure`; the counterpart of turbomind::Metric (metric.h:13-54). */
+typedef struct w4a16_metric {
+    int   id;          /* algo_id accepted by w4a16_gemm                        */
+    int   feasible;    /* 1 if the kernel can run this shape                    */
+    int   best;        /* 1 for the algo the heuristic (algo_id < 0) would pick */
+    int   kind;        /* 0 = decode (skinny) kernel, 1 = MFMA prefill kernel   */
+    int   tile_n;      /* output features per workgroup                         */
+    int   tile_t;      /* tokens per workgroup                                  */
+    int   slices;      /* K-slices (waves along K) per workgroup                */
+    int   grid;        /* workgroups launched                                   */
+    float ms;          /* total time of `count` launches, +inf if not feasible  */
+    int   count;       /* number of timed launches                              */
+} w4a16_metric;
+
+/* GemmS4F16::GemmS4F16 / ~GemmS4F16 (gemm_s4_f16.h:19-21, gemm_s4_f16.cu:236-252).
+ * The handle owns two events and nothing else; it binds to the current device. */
+int  w4a16_create(w4a16_handle** out);
+void w4a16_destroy(w4a16_handle* h);
+
+/* GemmS4F16::Run (gemm_s4_f16.h:41-51, gemm_s4_f16.cu:208-234,284-297).
+ *   C  fp16 [tokens, n_out]  (W4A16_FUSED_SILU_FFN: [tokens, n_out/2])
+ *   A  repacked int4 weights from w4a16_convert_s4_k_m8, k*n_out/2 bytes
+ *   X  fp16 [tokens, k] row-major (the reference's B)
+ *   Q  half2 [k/group_size, n_out] from w4a16_convert_s4_k_m8
+ *   R  fp16 [tokens, n_out] residual, W4A16_FUSED_ADD only (may alias C), else NULL
+ * Computes C = epilogue(X * dequant(A, Q)) with fp32 accumulation:
+ *   W4A16_GEMM            C[t,n] = fp16(acc[t,n])                      (gemm_s4_f16.cu:22-29)
+ *   W4A16_FUSED_SILU_FFN  g = fp16(acc[t,2j]), u = fp16(acc[t,2j+1]);
+ *                         C[t,j] = fp16(g / (1 + exp(-g)) * u)         (gemm_s4_f16.cu:31-42)
+ *   W4A16_FUSED_ADD       C[t,n] = fp16(float(R[t,n]) + float(fp16(acc[t,n])))
+ *                         (no counterpart in GemmS4F16; the add of
+ *                          llama_decoder_kernels.cu:52-57 applied as in LlamaDecoder.cc:228-235)
+ * algo_id < 0 selects a kernel by heuristic (gemm_s4_f16.cu:184-206 `Estimate`).
+ * Requires group_size == 128, k % 128 == 0, n_out % 16 == 0, tokens >= 0. */
+int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R,
+               int n_out, int tokens, int k, int group_size, int epilogue, int algo_id, void* stream);
+
+/* GemmS4F16::Measure (gemm_s4_f16.h:29-39, gemm_s4_f16.cu:98-169): times every feasible
+ * kernel (10 warm-up + 100 timed launches each) and writes up to `capacity` rows sorted
+ * by time; returns the number of rows, or a negative error.  Synchronises `stream`. */
+int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R,
+                  int n_out, int tokens, int k, int group_size, int epilogue,
+                  w4a16_metric* metrics, int capacity, void* stream);
+
+/* Number of kernels `w4a16_gemm` can dispatch to (valid algo_id are 0 .. count-1). */
+int w4a16_algo_count(void);
+
+/* convert_s4_k_m8 (format.h:15-24, format.cu:97-113).  Inputs are the AWQ tensors
+ *   A_src  uint32 [k, m/8], qzeros uint32 [k/group_size, m/8], scales fp16 [k/group_size, m]
+ * (pack order of lmdeploy/pytorch/modules/linear.py:85,105-108).  Outputs
+ *   A_dst  uint32 [k*m/8]  weights in the gfx950 tiled layout (same byte count as A_src)
+ *   Q_dst  half2  [k/group_size, m] = (64 + zero, scale), bit-identical to the reference's
+ * `workspace` (k/group_size*m halves) is accepted for signature compatibility and unused.
+ * m = output features, must be a multiple of 16; k a multiple of 128. */
+int w4a16_convert_s4_k_m8(uint32_t* A_dst, void* Q_dst, void* workspace, const uint32_t* A_src,
+                          const void* scales, const uint32_t* qzeros, int m, int k, int group_size,
+                          void* stream);
+
+/* reformat_s4_k_m8 (format.h:13, format.cu:69-75): the weight half of the conversion alone,
+ * AWQ words [k, m/8] -> the tiled layout the GEMM kernels read (here the gfx950 one).
+ * format.h:11 `reformat_s4_k8_m` is an unused alternative layout and has no counterpart. */
+int w4a16_reformat_s4_k_m8(uint32_t* dst, const uint32_t* src, int m, int k, void* stream);
+
+/* fuse_w1_w3_s4_k_m8 (format.h:28, format.cu:123-130): AWQ-packed cat(w1, w3) [2, k, m/8]
+ * -> AWQ-packed [k, 2m/8] with logical column 2j = w1[:, j], 2j+1 = w3[:, j]. */
+int w4a16_fuse_w1_w3_s4_k_m8(uint32_t* dst, const uint32_t* src, int m, int k, void* stream);
+
+/* transpose_qk_s4_k_m8_hf (format.h:26, format.cu:115-121): AWQ-packed [k, m/8]; within
+ * every head of size_per_head columns, dst column 2i+r = src column r*size_per_head/2 + i. */
+int w4a16_transpose_qk_s4_k_m8_hf(uint32_t* dst, const uint32_t* src, int m, int k, int size_per_head,
+                                  void* stream);
+
+/* dequantize_s4 (format.h:30, format.cu:132-142): `count` AWQ words -> 8*count fp16 holding
+ * the raw nibble values in logical column order.  Runs on `stream` (the reference ignores it). */
+int w4a16_dequantize_s4(void* dst, const uint32_t* src, size_t count, void* stream);
+
+/* Inverse of w4a16_convert_s4_k_m8 (no counterpart in the reference; exists so that the
+ * repack can be checked bit for bit): recovers the AWQ tensors from (A, Q).  Any of the
+ * three outputs may be NULL. */
+int w4a16_unpack_repacked(uint32_t* qweight, uint32_t* qzeros, void* scales, const uint32_t* A,
+                          const void* Q, int m, int k, int group_size, void* stream);
+
+/* Dequantised weights W fp16 [k, m] row-major from (A, Q), computed exactly as the
+ * reference kernel does (common.h:218-235): W = mul.ftz(sub.ftz(64+q, 64+z), s). */
+int w4a16_dequantize_repacked(void* W, const uint32_t* A, const void* Q, int m, int k, int group_size,
+                              void* stream);
+
+/* Converts weights already in the REFERENCE's tiled layout (output of its
+ * convert_s4_k_m8, i.e. a `.qweight` file written by deploy.py:142-146) to the gfx950
+ * layout.  Q needs no conversion.  m % 32 == 0, k % 128 == 0. */
+int w4a16_from_reference_layout(uint32_t* A_dst, const uint32_t* A_ref, int m, int k, void* stream);
+
+const char* w4a16_last_error(void);
+const char* w4a16_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* W4A16_H_ */

@@ -1,0 +1,67 @@
+"""ctypes binding of libw4a16.so.  There is no fallback: if the library is missing or lacks a
+symbol, importing fails loudly."""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_size_t, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libw4a16.so")
+
+OK, EGROUP, ESHAPE, EHIP, EARG, EALGO = 0, -1, -2, -3, -4, -5
+GEMM, FUSED_SILU_FFN, FUSED_ADD = 0, 1, 2
+
+
+class Metric(Structure):
+    """struct w4a16_metric of include/w4a16.h."""
+    _fields_ = [("id", c_int), ("feasible", c_int), ("best", c_int), ("kind", c_int), ("tile_n", c_int),
+                ("tile_t", c_int), ("slices", c_int), ("grid", c_int), ("ms", c_float), ("count", c_int)]
+
+
+class W4A16Error(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(message)
+        self.code = code
+
+
+# every symbol that include/w4a16.h declares: (restype, argtypes)
+SIGNATURES = {
+    "w4a16_create": (c_int, [POINTER(c_void_p)]),
+    "w4a16_destroy": (None, [c_void_p]),
+    "w4a16_gemm": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_void_p]),
+    "w4a16_measure": (c_int, [c_void_p] * 6 + [c_int] * 5 + [POINTER(Metric), c_int, c_void_p]),
+    "w4a16_algo_count": (c_int, []),
+    "w4a16_convert_s4_k_m8": (c_int, [c_void_p] * 6 + [c_int] * 3 + [c_void_p]),
+    "w4a16_reformat_s4_k_m8": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "w4a16_fuse_w1_w3_s4_k_m8": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "w4a16_transpose_qk_s4_k_m8_hf": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "w4a16_dequantize_s4": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "w4a16_unpack_repacked": (c_int, [c_void_p] * 5 + [c_int] * 3 + [c_void_p]),
+    "w4a16_dequantize_repacked": (c_int, [c_void_p] * 3 + [c_int] * 3 + [c_void_p]),
+    "w4a16_from_reference_layout": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "w4a16_last_error": (c_char_p, []),
+    "w4a16_version": (c_char_p, []),
+}
+
+
+def _load() -> ctypes.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "%s not found: build it with `python -m lmdeploy_amd.build` (needs hipcc); "
+            "there is no CPU fallback" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is missing
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+
+
+def check(code: int) -> int:
+    if code < 0:
+        raise W4A16Error(code, lib.w4a16_last_error().decode())
+    return code

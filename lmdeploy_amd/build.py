@@ -1,0 +1,84 @@
+"""Builds libw4a16.so (HIP kernels for gfx950 + the C ABI) in-tree with hipcc.
+
+Usage: python -m lmdeploy_amd.build            (or build_library() from Python)
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_DIR = os.path.join(HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libw4a16.so")
+
+SOURCES = ["api.cpp", "repack.hip", "gemm_decode.hip", "gemm_prefill.hip"]
+
+# -packed-fp32-ops off: hipcc must not form v_pk_*_f32 instructions for this target.
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; ROCm is required to build libw4a16.so")
+    return exe
+
+
+def _compile(src: str, obj_dir: str) -> str:
+    obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+    cmd = [_hipcc(), *HIP_FLAGS]
+    if src.endswith(".cpp"):
+        cmd += ["-x", "hip"]
+    cmd += ["-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
+    return obj
+
+
+def build_library(verbose: bool = True) -> str:
+    """Compiles every source and links the shared library; always rebuilds."""
+    obj_dir = os.path.join(HERE, "build")
+    os.makedirs(obj_dir, exist_ok=True)
+    os.makedirs(LIB_DIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
+        objs = list(ex.map(lambda s: _compile(s, obj_dir), SOURCES))
+    tmp = LIB_PATH + ".tmp"
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
+    os.replace(tmp, LIB_PATH)
+    if verbose:
+        print("built", LIB_PATH, os.path.getsize(LIB_PATH), "bytes")
+    return LIB_PATH
+
+
+def check_headers(verbose: bool = True) -> str:
+    """Compiles and links tests/cpp/llama_linear_dropin.cpp against the C++ front-end headers and
+    the library: the proof that a LlamaLinear-shaped caller builds against them."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "cpp", "llama_linear_dropin.cpp")
+    out = os.path.join(HERE, "build", "llama_linear_dropin")
+    os.makedirs(os.path.dirname(out), exist_ok=True)
+    cmd = [_hipcc(), "-x", "hip", "--offload-arch=gfx950", "-std=c++17", "-O1", "-Wall",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I", os.path.join(root, "include"), src, "-o", out, "-L", LIB_DIR, "-lw4a16",
+           "-Wl,-rpath," + LIB_DIR]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("drop-in header check failed:\n%s\n%s" % (r.stdout, r.stderr))
+    if verbose:
+        print("built", out)
+    return out
+
+
+if __name__ == "__main__":
+    build_library()
+    check_headers()
+    sys.exit(0)

@@ -1,0 +1,370 @@
+// The C ABI of libw4a16.so: argument validation, kernel selection, timing and error
+// reporting.  No kernel code lives here.
+#include "../../include/w4a16.h"
+#include "w4a16_internal.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <limits>
+#include <vector>
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what)
+{
+    return fail(W4A16_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+bool aligned16(const void* p)
+{
+    return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+}  // namespace
+
+struct w4a16_handle {
+    hipEvent_t ev_start{};
+    hipEvent_t ev_end{};
+    int        device{};
+};
+
+namespace w4a16 {
+
+// ---- kernel table (the counterpart of the 17 GemmKernel objects of gemm_s4_f16.cu:72-93) ----
+namespace {
+
+std::vector<Algo> build_table()
+{
+    std::vector<Algo> t;
+    for (int r : {1, 2, 4})
+        for (int s : {1, 2, 4, 8, 16}) {
+            if (r == 4 && s == 16) continue;
+            t.push_back(Algo{0, 16 * r, 16, s, r});
+        }
+    for (int v = 0; v < prefill_variants(); ++v) {
+        int tn = 0, tt = 0;
+        prefill_tile(v, tn, tt);
+        t.push_back(Algo{1, tn, tt, 1, v});
+    }
+    return t;
+}
+
+const std::vector<Algo>& table()
+{
+    static const std::vector<Algo> t = build_table();
+    return t;
+}
+
+}  // namespace
+
+int algo_count()
+{
+    return (int)table().size();
+}
+
+const Algo& algo_at(int id)
+{
+    return table()[id];
+}
+
+bool algo_feasible(int id, int N, int T, int K)
+{
+    const Algo& a = algo_at(id);
+    return a.kind == 0 ? decode_feasible(a.param, a.slices, N, T, K) : prefill_feasible(a.param, N, T, K);
+}
+
+int algo_grid(int id, int N, int T, int K)
+{
+    const Algo& a = algo_at(id);
+    return a.kind == 0 ? decode_grid(a.param, a.slices, N, T, K) : prefill_grid(a.param, N, T, K);
+}
+
+hipError_t algo_launch(int id, const GemmArgs& g, hipStream_t st)
+{
+    const Algo& a = algo_at(id);
+    return a.kind == 0 ? decode_launch(a.param, a.slices, g, st) : prefill_launch(a.param, g, st);
+}
+
+// Heuristic choice.  Few tokens: the decode kernel, with enough K slices that the chip holds
+// about eight waves per CU and each wave still owns two or more quantisation groups; two
+// column tiles per wave once more than eight tokens share the activations.  Many tokens: the
+// MFMA prefill kernel whose tile count wastes the least of the last wave of workgroups.
+int algo_pick(int N, int T, int K)
+{
+    const int G = K / 128;
+    if (T <= 0 || N <= 0 || K <= 0) return -1;
+    int best = -1;
+    if (T >= 64) {
+        double best_cost = std::numeric_limits<double>::infinity();
+        for (int id = 0; id < algo_count(); ++id) {
+            const Algo& a = algo_at(id);
+            if (a.kind != 1 || !algo_feasible(id, N, T, K)) continue;
+            const double grid   = algo_grid(id, N, T, K);
+            const double rounds = std::ceil(grid / 256.0);
+            // time ~ rounds * work per tile, with a mild bonus for larger tiles (operand reuse)
+            const double per_tile = (double)a.tile_n * a.tile_t;
+            const double padded_t = std::ceil((double)T / a.tile_t) * a.tile_t / T;
+            const double cost = rounds * per_tile * padded_t * (1.0 + 24.0 / a.tile_n + 24.0 / a.tile_t);
+            if (cost < best_cost) {
+                best_cost = cost;
+                best      = id;
+            }
+        }
+        if (best >= 0) return best;
+    }
+    const int want_r = T > 8 && N % 32 == 0 ? 2 : 1;
+    for (int r = want_r; r >= 1 && best < 0; r >>= 1) {
+        const long tiles = (long)(N / (16 * r)) * ((T + 15) / 16);
+        int        s     = 16;
+        while (s > 1 && (tiles * s > 4096 || G / s < 2)) s >>= 1;
+        for (int id = 0; id < algo_count(); ++id) {
+            const Algo& a = algo_at(id);
+            if (a.kind == 0 && a.param == r && a.slices == s && algo_feasible(id, N, T, K)) {
+                best = id;
+                break;
+            }
+        }
+    }
+    if (best >= 0) return best;
+    for (int id = 0; id < algo_count(); ++id)
+        if (algo_feasible(id, N, T, K)) return id;
+    return -1;
+}
+
+}  // namespace w4a16
+
+using namespace w4a16;
+
+namespace {
+
+int check_gemm_args(const w4a16_handle* h, const void* C, const void* A, const void* X, const void* Q,
+                    const void* R, int n_out, int tokens, int k, int group_size, int epilogue)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
+    if (epilogue < W4A16_GEMM || epilogue > W4A16_FUSED_ADD) return fail(W4A16_EARG, "unknown epilogue %d", epilogue);
+    if (n_out < 0 || tokens < 0 || k < 0) return fail(W4A16_EARG, "negative size");
+    if (tokens == 0 || n_out == 0) return 1;  // nothing to do
+    if (!C || !A || !X || !Q) return fail(W4A16_EARG, "null pointer");
+    if (epilogue == W4A16_FUSED_ADD && !R) return fail(W4A16_EARG, "fused add needs a residual");
+    if (!aligned16(A) || !aligned16(X) || (reinterpret_cast<uintptr_t>(C) & 3u) ||
+        (reinterpret_cast<uintptr_t>(Q) & 3u) || (R && (reinterpret_cast<uintptr_t>(R) & 3u)))
+        return fail(W4A16_EARG, "misaligned pointer (A and X need 16 bytes, C, Q, R need 4)");
+    if (k == 0 || k % 128 != 0 || n_out % 16 != 0) return fail(W4A16_ESHAPE, "no feasible kernel found");
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int w4a16_create(w4a16_handle** out)
+{
+    if (!out) return fail(W4A16_EARG, "null output pointer");
+    *out = nullptr;
+    auto*      h = new w4a16_handle();
+    hipError_t e = hipGetDevice(&h->device);
+    if (e == hipSuccess) e = hipEventCreate(&h->ev_start);
+    if (e == hipSuccess) e = hipEventCreate(&h->ev_end);
+    if (e != hipSuccess) {
+        if (h->ev_start) (void)hipEventDestroy(h->ev_start);
+        delete h;
+        return hip_fail(e, "w4a16_create");
+    }
+    *out = h;
+    return W4A16_OK;
+}
+
+void w4a16_destroy(w4a16_handle* h)
+{
+    if (!h) return;
+    (void)hipEventDestroy(h->ev_end);
+    (void)hipEventDestroy(h->ev_start);
+    delete h;
+}
+
+int w4a16_algo_count(void)
+{
+    return algo_count();
+}
+
+int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R, int n_out,
+               int tokens, int k, int group_size, int epilogue, int algo_id, void* stream)
+{
+    const int chk = check_gemm_args(h, C, A, X, Q, R, n_out, tokens, k, group_size, epilogue);
+    if (chk < 0) return chk;
+    if (chk > 0) return W4A16_OK;
+    if (algo_id >= algo_count()) return fail(W4A16_EALGO, "algo_id %d out of range (0..%d)", algo_id, algo_count() - 1);
+    if (algo_id < 0) algo_id = algo_pick(n_out, tokens, k);
+    if (algo_id < 0 || !algo_feasible(algo_id, n_out, tokens, k)) return fail(W4A16_ESHAPE, "no feasible kernel found");
+    GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
+               n_out,        tokens,             k,                  epilogue};
+    const hipError_t e = algo_launch(algo_id, g, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "w4a16_gemm launch");
+    return W4A16_OK;
+}
+
+int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R, int n_out,
+                  int tokens, int k, int group_size, int epilogue, w4a16_metric* metrics, int capacity, void* stream)
+{
+    const int chk = check_gemm_args(h, C, A, X, Q, R, n_out, tokens, k, group_size, epilogue);
+    if (chk < 0) return chk;
+    if (!metrics || capacity <= 0) return fail(W4A16_EARG, "no room for metrics");
+    if (chk > 0) return 0;
+    constexpr int kWarmup = 10, kMeasure = 100;  // gemm_s4_f16.cu:258-259
+    hipStream_t   st   = (hipStream_t)stream;
+    const int     best = algo_pick(n_out, tokens, k);
+    GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
+               n_out,        tokens,             k,                  epilogue};
+    std::vector<w4a16_metric> all;
+    for (int id = 0; id < algo_count(); ++id) {
+        const Algo&  a = algo_at(id);
+        w4a16_metric m{};
+        m.id       = id;
+        m.kind     = a.kind;
+        m.tile_n   = a.tile_n;
+        m.tile_t   = a.tile_t;
+        m.slices   = a.slices;
+        m.best     = id == best;
+        m.feasible = algo_feasible(id, n_out, tokens, k);
+        m.count    = 1;
+        m.ms       = std::numeric_limits<float>::infinity();
+        if (m.feasible) {
+            m.grid = algo_grid(id, n_out, tokens, k);
+            for (int j = 0; j < kWarmup + kMeasure; ++j) {
+                if (j == kWarmup) (void)hipEventRecord(h->ev_start, st);
+                const hipError_t e = algo_launch(id, g, st);
+                if (e != hipSuccess) return hip_fail(e, "w4a16_measure launch");
+            }
+            (void)hipEventRecord(h->ev_end, st);
+            hipError_t e = hipEventSynchronize(h->ev_end);
+            if (e != hipSuccess) return hip_fail(e, "w4a16_measure sync");
+            float ms = 0.f;
+            e        = hipEventElapsedTime(&ms, h->ev_start, h->ev_end);
+            if (e != hipSuccess) return hip_fail(e, "w4a16_measure elapsed");
+            m.ms    = ms;
+            m.count = kMeasure;
+        }
+        all.push_back(m);
+    }
+    std::stable_sort(all.begin(), all.end(), [](const w4a16_metric& a, const w4a16_metric& b) { return a.ms < b.ms; });
+    const int n = std::min<int>(capacity, (int)all.size());
+    std::memcpy(metrics, all.data(), sizeof(w4a16_metric) * n);
+    return n;
+}
+
+static int check_repack(const char* what, int m, int k, int m_mult, int k_mult)
+{
+    if (m < 0 || k < 0) return fail(W4A16_EARG, "%s: negative size", what);
+    if (m % m_mult != 0 || k % k_mult != 0)
+        return fail(W4A16_ESHAPE, "%s: m must be a multiple of %d and k of %d (got m=%d k=%d)", what, m_mult, k_mult, m, k);
+    return 0;
+}
+
+int w4a16_convert_s4_k_m8(uint32_t* A_dst, void* Q_dst, void* workspace, const uint32_t* A_src, const void* scales,
+                          const uint32_t* qzeros, int m, int k, int group_size, void* stream)
+{
+    (void)workspace;
+    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
+    if (int c = check_repack("convert_s4_k_m8", m, k, 16, 128)) return c;
+    if (m == 0 || k == 0) return W4A16_OK;
+    if (!A_dst || !Q_dst || !A_src || !scales || !qzeros) return fail(W4A16_EARG, "convert_s4_k_m8: null pointer");
+    const hipError_t e = launch_convert(A_dst, (uint32_t*)Q_dst, A_src, (const uint16_t*)scales, qzeros, m, k,
+                                        (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "convert_s4_k_m8");
+}
+
+int w4a16_reformat_s4_k_m8(uint32_t* dst, const uint32_t* src, int m, int k, void* stream)
+{
+    if (int c = check_repack("reformat_s4_k_m8", m, k, 16, 128)) return c;
+    if (m == 0 || k == 0) return W4A16_OK;
+    if (!dst || !src) return fail(W4A16_EARG, "reformat_s4_k_m8: null pointer");
+    const hipError_t e = launch_convert(dst, nullptr, src, nullptr, nullptr, m, k, (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "reformat_s4_k_m8");
+}
+
+int w4a16_fuse_w1_w3_s4_k_m8(uint32_t* dst, const uint32_t* src, int m, int k, void* stream)
+{
+    if (int c = check_repack("fuse_w1_w3_s4_k_m8", m, k, 8, 1)) return c;
+    if (m == 0 || k == 0) return W4A16_OK;
+    if (!dst || !src) return fail(W4A16_EARG, "fuse_w1_w3_s4_k_m8: null pointer");
+    const hipError_t e = launch_fuse_w1_w3(dst, src, m, k, (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "fuse_w1_w3_s4_k_m8");
+}
+
+int w4a16_transpose_qk_s4_k_m8_hf(uint32_t* dst, const uint32_t* src, int m, int k, int size_per_head, void* stream)
+{
+    if (size_per_head <= 0 || size_per_head % 2 != 0) return fail(W4A16_ESHAPE, "transpose_qk: bad size_per_head");
+    if (int c = check_repack("transpose_qk_s4_k_m8_hf", m, k, 8, 1)) return c;
+    if (m % size_per_head != 0) return fail(W4A16_ESHAPE, "transpose_qk: m is not a multiple of size_per_head");
+    if (m == 0 || k == 0) return W4A16_OK;
+    if (!dst || !src) return fail(W4A16_EARG, "transpose_qk_s4_k_m8_hf: null pointer");
+    const hipError_t e = launch_transpose_qk(dst, src, m, k, size_per_head, (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "transpose_qk_s4_k_m8_hf");
+}
+
+int w4a16_dequantize_s4(void* dst, const uint32_t* src, size_t count, void* stream)
+{
+    if (count == 0) return W4A16_OK;
+    if (!dst || !src) return fail(W4A16_EARG, "dequantize_s4: null pointer");
+    if (!aligned16(dst)) return fail(W4A16_EARG, "dequantize_s4: dst needs 16-byte alignment");
+    const hipError_t e = launch_dequantize_s4(dst, src, count, (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "dequantize_s4");
+}
+
+int w4a16_unpack_repacked(uint32_t* qweight, uint32_t* qzeros, void* scales, const uint32_t* A, const void* Q, int m,
+                          int k, int group_size, void* stream)
+{
+    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
+    if (int c = check_repack("unpack_repacked", m, k, 16, 128)) return c;
+    if (m == 0 || k == 0) return W4A16_OK;
+    if ((qweight && !A) || ((qzeros || scales) && !Q)) return fail(W4A16_EARG, "unpack_repacked: null pointer");
+    const hipError_t e = launch_unpack(qweight, qzeros, (uint16_t*)scales, A, (const uint32_t*)Q, m, k,
+                                       (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "unpack_repacked");
+}
+
+int w4a16_dequantize_repacked(void* W, const uint32_t* A, const void* Q, int m, int k, int group_size, void* stream)
+{
+    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
+    if (int c = check_repack("dequantize_repacked", m, k, 16, 128)) return c;
+    if (m == 0 || k == 0) return W4A16_OK;
+    if (!W || !A || !Q) return fail(W4A16_EARG, "dequantize_repacked: null pointer");
+    const hipError_t e = launch_dequantize_repacked((uint16_t*)W, A, (const uint32_t*)Q, m, k, (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "dequantize_repacked");
+}
+
+int w4a16_from_reference_layout(uint32_t* A_dst, const uint32_t* A_ref, int m, int k, void* stream)
+{
+    if (int c = check_repack("from_reference_layout", m, k, 32, 128)) return c;
+    if (m == 0 || k == 0) return W4A16_OK;
+    if (!A_dst || !A_ref) return fail(W4A16_EARG, "from_reference_layout: null pointer");
+    const hipError_t e = launch_from_reference(A_dst, A_ref, m, k, (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "from_reference_layout");
+}
+
+const char* w4a16_last_error(void)
+{
+    return g_err;
+}
+
+const char* w4a16_version(void)
+{
+    return "w4a16-gfx950 0.1";
+}
+
+}  // extern "C"

@@ -1,0 +1,63 @@
+// Internal C++ interface between the C ABI (api.hip) and the kernel launchers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace w4a16 {
+
+enum Epilogue { kEpiGemm = 0, kEpiSilu = 1, kEpiAdd = 2 };
+
+struct GemmArgs {
+    uint16_t*       C;   // fp16 out [T, N] or [T, N/2]
+    const uint32_t* A;   // tiled int4 weights
+    const uint16_t* X;   // fp16 [T, K]
+    const uint32_t* Q;   // half2 [K/128, N]
+    const uint16_t* R;   // fp16 residual [T, N] or null
+    int             N, T, K;
+    int             epilogue;
+};
+
+// One dispatchable kernel configuration.
+struct Algo {
+    int kind;     // 0 decode, 1 prefill
+    int tile_n;   // output features per workgroup
+    int tile_t;   // tokens per workgroup
+    int slices;   // waves along K per workgroup (decode) / 1
+    int param;    // kernel-specific variant index
+};
+
+int         algo_count();
+const Algo& algo_at(int id);
+// true if algo `id` can run the shape
+bool algo_feasible(int id, int N, int T, int K);
+// heuristic choice (the counterpart of Estimate); -1 if nothing is feasible
+int algo_pick(int N, int T, int K);
+// workgroups the launch would use
+int algo_grid(int id, int N, int T, int K);
+hipError_t algo_launch(int id, const GemmArgs& a, hipStream_t st);
+
+hipError_t launch_convert(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* A_src, const uint16_t* scales,
+                          const uint32_t* qzeros, int m, int k, hipStream_t st);
+hipError_t launch_unpack(uint32_t* qweight, uint32_t* qzeros, uint16_t* scales, const uint32_t* A,
+                         const uint32_t* Q, int m, int k, hipStream_t st);
+hipError_t launch_dequantize_repacked(uint16_t* W, const uint32_t* A, const uint32_t* Q, int m, int k,
+                                      hipStream_t st);
+hipError_t launch_dequantize_s4(void* dst, const uint32_t* src, size_t count, hipStream_t st);
+hipError_t launch_fuse_w1_w3(uint32_t* dst, const uint32_t* src, int m, int k, hipStream_t st);
+hipError_t launch_transpose_qk(uint32_t* dst, const uint32_t* src, int m, int k, int size_per_head, hipStream_t st);
+hipError_t launch_from_reference(uint32_t* dst, const uint32_t* ref, int m, int k, hipStream_t st);
+
+// decode (skinny) kernels: R column tiles per wave x S waves along K
+bool       decode_feasible(int r, int s, int N, int T, int K);
+int        decode_grid(int r, int s, int N, int T, int K);
+hipError_t decode_launch(int r, int s, const GemmArgs& a, hipStream_t st);
+
+// MFMA prefill kernels
+int        prefill_variants();
+void       prefill_tile(int variant, int& tile_n, int& tile_t);
+bool       prefill_feasible(int variant, int N, int T, int K);
+int        prefill_grid(int variant, int N, int T, int K);
+hipError_t prefill_launch(int variant, const GemmArgs& a, hipStream_t st);
+
+}  // namespace w4a16

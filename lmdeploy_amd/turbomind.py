@@ -1,0 +1,126 @@
+"""Host-side mirror of the reference's interface to the W4A16 path.
+
+* the four repack functions that `src/turbomind/python/bind.cpp:414-465` exports from
+  `_turbomind` and `lmdeploy/serve/turbomind/deploy.py:631-665` calls, with the same names
+  and argument order, taking torch tensors on the GPU;
+* `GemmS4F16`, the operator of `src/turbomind/kernels/gemm_s_f16/gemm_s4_f16.h:17-56`.
+
+Sizes follow the reference: `m` = output features, `k` = input features, `n` = tokens.
+All work is queued on torch's current stream.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional
+
+import torch
+
+from . import _lib
+from ._lib import Metric, W4A16Error, check, lib  # noqa: F401
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise ValueError("tensor must live on the GPU")
+    if not t.is_contiguous():
+        raise ValueError("tensor must be contiguous")
+    return t.data_ptr()
+
+
+def convert_s4_k_m8(A_dst, Q_dst, ws, A_src, scales, qzeros, m: int, k: int, group_size: int) -> None:
+    """bind.cpp:431-456.  A_src int32 [k, m/8], scales fp16 [k/g, m], qzeros int32 [k/g, m/8] ->
+    A_dst (same bytes as A_src, gfx950 tiled layout), Q_dst int32 [k/g, m] = half2(64 + zero, scale)."""
+    if A_src.numel() * 8 != m * k or A_dst.numel() != A_src.numel():
+        raise ValueError("qweight shape does not match m, k")
+    g = k // group_size if group_size > 0 else 0
+    if scales.numel() != g * m or qzeros.numel() * 8 != g * m or Q_dst.numel() * Q_dst.element_size() != g * m * 4:
+        raise ValueError("scales / qzeros / Q shape does not match m, k, group_size")
+    check(lib.w4a16_convert_s4_k_m8(_ptr(A_dst), _ptr(Q_dst), _ptr(ws), _ptr(A_src), _ptr(scales), _ptr(qzeros),
+                                    m, k, group_size, _stream()))
+
+
+def fuse_w1_w3_s4_k_m8(src, dst, m: int, k: int) -> None:
+    """bind.cpp:424-429.  src = cat(w1, w3) int32 [2k, m/8] -> dst [k, 2m/8], columns interleaved."""
+    if src.numel() * 8 != 2 * m * k or dst.numel() != src.numel():
+        raise ValueError("shape does not match m, k")
+    check(lib.w4a16_fuse_w1_w3_s4_k_m8(_ptr(dst), _ptr(src), m, k, _stream()))
+
+
+def transpose_qk_s4_k_m8(src, dst, m: int, k: int, size_per_head: int) -> None:
+    """bind.cpp:414-422.  Rotary re-ordering of the q/k columns of an AWQ-packed [k, m/8] tensor."""
+    if src.numel() * 8 != m * k or dst.numel() != src.numel():
+        raise ValueError("shape does not match m, k")
+    check(lib.w4a16_transpose_qk_s4_k_m8_hf(_ptr(dst), _ptr(src), m, k, size_per_head, _stream()))
+
+
+def dequantize_s4(src, dst) -> None:
+    """bind.cpp:458-465.  int32 words -> fp16 raw nibble values (8 per word)."""
+    if src.numel() * 8 != dst.numel():
+        raise ValueError("FT_CHECK(src_count * 8 == dst_count) failed")
+    check(lib.w4a16_dequantize_s4(_ptr(dst), _ptr(src), src.numel(), _stream()))
+
+
+def unpack_repacked(A, Q, m: int, k: int, group_size: int = 128):
+    """Inverse of convert_s4_k_m8: returns (qweight, qzeros, scales) as the AWQ tensors."""
+    g = k // group_size
+    qweight = torch.empty((k, m // 8), dtype=torch.int32, device=A.device)
+    qzeros = torch.empty((g, m // 8), dtype=torch.int32, device=A.device)
+    scales = torch.empty((g, m), dtype=torch.float16, device=A.device)
+    check(lib.w4a16_unpack_repacked(_ptr(qweight), _ptr(qzeros), _ptr(scales), _ptr(A), _ptr(Q), m, k, group_size,
+                                    _stream()))
+    return qweight, qzeros, scales
+
+
+def dequantize_repacked(A, Q, m: int, k: int, group_size: int = 128):
+    """fp16 W[k, m] with the reference kernel's arithmetic: fp16((q - z) * s)."""
+    W = torch.empty((k, m), dtype=torch.float16, device=A.device)
+    check(lib.w4a16_dequantize_repacked(_ptr(W), _ptr(A), _ptr(Q), m, k, group_size, _stream()))
+    return W
+
+
+def from_reference_layout(A_ref, m: int, k: int):
+    """Weights in the reference's own tiled layout -> the gfx950 layout."""
+    out = torch.empty_like(A_ref)
+    check(lib.w4a16_from_reference_layout(_ptr(out), _ptr(A_ref), m, k, _stream()))
+    return out
+
+
+class GemmS4F16:
+    """gemm_s4_f16.h:17-56.  `Run(C, A, B, Q, m, n, k, group_size, type, algo_id)` with m = output
+    features, n = tokens; B is the fp16 activation matrix [n, k]."""
+    kGemm = _lib.GEMM
+    kFusedSiluFfn = _lib.FUSED_SILU_FFN
+    kFusedAdd = _lib.FUSED_ADD  # extension: C = residual + gemm
+
+    def __init__(self):
+        h = ctypes.c_void_p()
+        check(lib.w4a16_create(ctypes.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            lib.w4a16_destroy(h)
+
+    def Run(self, C, A, B, Q, m: int, n: int, k: int, group_size: int, type: int = 0, algo_id: int = -1,
+            residual=None, stream: Optional[int] = None) -> None:
+        check(lib.w4a16_gemm(self._h, _ptr(C), _ptr(A), _ptr(B), _ptr(Q), _ptr(residual), m, n, k, group_size, type,
+                             algo_id, _stream() if stream is None else stream))
+
+    def Measure(self, C, A, B, Q, m: int, n: int, k: int, group_size: int, type: int = 0,
+                residual=None) -> List[Metric]:
+        cap = lib.w4a16_algo_count()
+        buf = (Metric * cap)()
+        cnt = check(lib.w4a16_measure(self._h, _ptr(C), _ptr(A), _ptr(B), _ptr(Q), _ptr(residual), m, n, k,
+                                      group_size, type, buf, cap, _stream()))
+        return [buf[i] for i in range(cnt)]
+
+    @staticmethod
+    def algo_count() -> int:
+        return lib.w4a16_algo_count()

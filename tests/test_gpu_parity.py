@@ -1,0 +1,281 @@
+"""GPU parity: the HIP library, called through its C ABI, against the CPU oracle.
+
+Integer work (repack, unpack, fuse, transpose, dequantised weights) must be bit exact.
+GEMM outputs must satisfy max|y - yref| / max|yref| <= 1e-2 in fp16 (the stated tolerance),
+and are exact in the special cases where the mathematics fixes the answer."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import w4a16_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def tm():
+    import lmdeploy_amd.turbomind as tm
+    return tm
+
+
+@pytest.fixture(scope="module")
+def gemm(tm):
+    return tm.GemmS4F16()
+
+
+def dev(a: np.ndarray) -> torch.Tensor:
+    if a.dtype == np.uint32:
+        a = a.view(np.int32)
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host_u32(t: torch.Tensor) -> np.ndarray:
+    return t.cpu().numpy().view(np.uint32)
+
+
+def convert(tm, d, N, K):
+    qw, qz, s = dev(d["qweight"]), dev(d["qzeros"]), dev(d["scales"])
+    A = torch.zeros_like(qw)
+    Q = torch.zeros_like(s, dtype=torch.int32)
+    ws = torch.zeros_like(s)
+    tm.convert_s4_k_m8(A, Q, ws, qw, s, qz, N, K, 128)
+    return A, Q
+
+
+def run(tm, gemm, d, A, Q, T, K, N, kind=0, algo=-1):
+    X = dev(d["X"])
+    R = dev(d["R"]) if kind == 2 else None
+    n_out = N // 2 if kind == 1 else N
+    C = torch.full((T, n_out), float("nan"), dtype=torch.float16, device="cuda")
+    gemm.Run(C, A, X, Q, N, T, K, 128, kind, algo, residual=R)
+    torch.cuda.synchronize()
+    return C.cpu().numpy()
+
+
+# ------------------------------------------------------------------ repack (integer, bit exact)
+@pytest.mark.parametrize("K,N", [(128, 16), (256, 48), (512, 4096), (4096, 4096), (11008, 4096), (4096, 22016)])
+def test_convert_bit_exact_and_round_trip(tm, K, N):
+    d = O.make_inputs(100 + K + N, 1, K, N)
+    A, Q = convert(tm, d, N, K)
+    A_ref, Q_ref = O.convert_s4_k_m8(d["qweight"], d["scales"], d["qzeros"], N, K, 128)
+    assert np.array_equal(host_u32(A).reshape(-1), A_ref)
+    assert np.array_equal(host_u32(Q), Q_ref)
+    qw, qz, s = tm.unpack_repacked(A, Q, N, K)
+    assert np.array_equal(host_u32(qw), d["qweight"])          # == the reference's own unpack of the input
+    assert np.array_equal(host_u32(qz), d["qzeros"])
+    assert np.array_equal(s.cpu().numpy().view(np.uint16), d["scales"].view(np.uint16))
+
+
+@pytest.mark.parametrize("K,N", [(256, 48), (4096, 4096), (11008, 4096)])
+def test_dequantised_weights_bit_exact(tm, K, N):
+    d = O.make_inputs(200 + K + N, 1, K, N)
+    A, Q = convert(tm, d, N, K)
+    W = tm.dequantize_repacked(A, Q, N, K).cpu().numpy()
+    W_ref = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], 128)
+    assert np.array_equal(W.view(np.uint16), W_ref.view(np.uint16))
+
+
+def test_dequantised_weights_flush_subnormals(tm):
+    K, N = 256, 32
+    d = O.make_inputs(7, 1, K, N)
+    s = d["scales"].copy()
+    s[0, :] = np.float16(2.0 ** -16)      # subnormal scale
+    s[1, :] = np.float16(2.0 ** -14)      # products with |q - z| >= 1 are normal, 0 stays 0
+    s[1, ::3] = np.float16(3.0e-5)        # subnormal scale again
+    d["scales"] = s
+    A, Q = convert(tm, d, N, K)
+    W = tm.dequantize_repacked(A, Q, N, K).cpu().numpy()
+    W_ref = O.dequant_from_awq(d["qweight"], d["qzeros"], s, 128)
+    assert np.array_equal(W.view(np.uint16), W_ref.view(np.uint16))
+
+
+def test_dequantize_s4_bit_exact(tm):
+    rng = np.random.default_rng(3)
+    words = rng.integers(0, 2 ** 32, size=4099, dtype=np.uint64).astype(np.uint32)
+    dst = torch.empty(words.size * 8, dtype=torch.float16, device="cuda")
+    tm.dequantize_s4(dev(words), dst)
+    torch.cuda.synchronize()
+    assert np.array_equal(dst.cpu().numpy(), O.dequantize_s4(words))
+    with pytest.raises(ValueError):
+        tm.dequantize_s4(dev(words), dst[:-8])
+
+
+@pytest.mark.parametrize("K,N1", [(16, 48), (4096, 11008)])
+def test_fuse_w1_w3(tm, K, N1):
+    rng = np.random.default_rng(4)
+    w1 = rng.integers(0, 16, size=(K, N1), dtype=np.uint8)
+    w3 = rng.integers(0, 16, size=(K, N1), dtype=np.uint8)
+    src = np.concatenate([O.awq_pack(w1), O.awq_pack(w3)])
+    dst = torch.zeros(K, 2 * N1 // 8, dtype=torch.int32, device="cuda")
+    tm.fuse_w1_w3_s4_k_m8(dev(src), dst, N1, K)
+    torch.cuda.synchronize()
+    got = host_u32(dst)
+    assert np.array_equal(got, O.fuse_w1_w3_s4_k_m8(src, N1, K))
+    U = O.awq_unpack(got)
+    assert np.array_equal(U[:, 0::2], w1) and np.array_equal(U[:, 1::2], w3)
+
+
+@pytest.mark.parametrize("K,N,D", [(8, 96, 32), (512, 4096, 128)])
+def test_transpose_qk(tm, K, N, D):
+    rng = np.random.default_rng(5)
+    w = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    src = O.awq_pack(w)
+    dst = torch.zeros(K, N // 8, dtype=torch.int32, device="cuda")
+    tm.transpose_qk_s4_k_m8(dev(src), dst, N, K, D)
+    torch.cuda.synchronize()
+    assert np.array_equal(host_u32(dst), O.transpose_qk_s4_k_m8_hf(src, N, K, D))
+
+
+@pytest.mark.parametrize("K,N", [(128, 32), (512, 4096)])
+def test_from_reference_layout(tm, K, N):
+    d = O.make_inputs(6, 1, K, N)
+    A_ref_layout, _ = O.convert_s4_k_m8_reference(d["qweight"], d["scales"], d["qzeros"], N, K, 128)
+    ours = tm.from_reference_layout(dev(A_ref_layout), N, K)
+    torch.cuda.synchronize()
+    assert np.array_equal(host_u32(ours).reshape(-1), O.repack_gfx950(d["qweight"], N, K))
+
+
+# ------------------------------------------------------------------ GEMM, every kernel
+def _algos(gemm):
+    return list(range(gemm.algo_count()))
+
+
+@pytest.mark.parametrize("T", [1, 3, 16, 17, 33, 125])
+def test_every_kernel_small_shape(tm, gemm, T):
+    K, N = 1024, 256
+    d = O.make_inputs(300 + T, T, K, N, residual=True)
+    A, Q = convert(tm, d, N, K)
+    want = {k: O.gemm_s4_f16(d["X"], d["qweight"], d["qzeros"], d["scales"], 128, k, d.get("R")) for k in (0, 1, 2)}
+    ran = 0
+    for algo in _algos(gemm):
+        for kind in (0, 1, 2):
+            try:
+                got = run(tm, gemm, d, A, Q, T, K, N, kind, algo)
+            except tm.W4A16Error as e:
+                assert e.code == -2, e     # infeasible for this shape is the only acceptable failure
+                continue
+            ran += 1
+            err = O.max_abs_rel(got, want[kind])
+            assert np.isfinite(got).all() and err <= TOL, (algo, kind, err)
+    assert ran >= 20
+
+
+def test_identity_activations_return_weights(tm, gemm):
+    # X = I  =>  Y == W.  The prefill kernels use the reference's exact fp16 weight, so they are
+    # bit exact; the decode kernels scale after the group sum: (q - z) * s rounded once from fp32,
+    # which is the same single rounding.
+    K, N = 256, 128
+    d = O.make_inputs(9, K, K, N)
+    d["X"] = np.eye(K, dtype=np.float16)
+    A, Q = convert(tm, d, N, K)
+    W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], 128)
+    for algo in _algos(gemm):
+        try:
+            got = run(tm, gemm, d, A, Q, K, K, N, 0, algo)
+        except tm.W4A16Error:
+            continue
+        assert np.array_equal(got.view(np.uint16), W.view(np.uint16)), algo
+
+
+def test_exact_integer_case_and_zero_weights(tm, gemm):
+    rng = np.random.default_rng(12)
+    T, K, N = 5, 512, 64
+    q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(K // 128, N), dtype=np.uint8)
+    s = (2.0 ** rng.integers(-3, 2, size=(K // 128, N))).astype(np.float16)
+    X = rng.integers(-3, 4, size=(T, K)).astype(np.float16)
+    d = dict(qweight=O.awq_pack(q), qzeros=O.awq_pack(z), scales=s, X=X)
+    A, Q = convert(tm, d, N, K)
+    want = O.gemm_s4_f16(X, d["qweight"], d["qzeros"], s, 128)
+    for algo in _algos(gemm):
+        try:
+            got = run(tm, gemm, d, A, Q, T, K, N, 0, algo)
+        except tm.W4A16Error:
+            continue
+        assert np.array_equal(got, want), algo
+    # q == z  =>  Y == 0 ; with the residual epilogue  =>  Y == R bit for bit
+    d0 = dict(d, qweight=O.awq_pack(np.repeat(z, 128, axis=0)), R=rng.standard_normal((T, N)).astype(np.float16))
+    A0, Q0 = convert(tm, d0, N, K)
+    assert not np.any(run(tm, gemm, d0, A0, Q0, T, K, N, 0))
+    assert np.array_equal(run(tm, gemm, d0, A0, Q0, T, K, N, 2).view(np.uint16), d0["R"].view(np.uint16))
+
+
+def test_residual_in_place(tm, gemm):
+    T, K, N = 8, 512, 128
+    d = O.make_inputs(21, T, K, N, residual=True)
+    A, Q = convert(tm, d, N, K)
+    want = O.gemm_s4_f16(d["X"], d["qweight"], d["qzeros"], d["scales"], 128, O.EPI_ADD, d["R"])
+    C = dev(d["R"])
+    gemm.Run(C, A, dev(d["X"]), Q, N, T, K, 128, gemm.kFusedAdd, -1, residual=C)   # C aliases R
+    torch.cuda.synchronize()
+    assert O.max_abs_rel(C.cpu().numpy(), want) <= TOL
+
+
+# ------------------------------------------------------------------ the benchmark configurations
+LLAMA7B = [("qkv", 4096, 12288, 0), ("o", 4096, 4096, 0), ("gate_up", 4096, 22016, 1), ("down", 11008, 4096, 2)]
+SEED = {"qkv": 11, "o": 22, "gate_up": 33, "down": 44}
+
+
+@pytest.mark.parametrize("name,K,N,kind", LLAMA7B)
+def test_llama7b_decode_shapes(tm, gemm, name, K, N, kind):
+    d = O.make_inputs(SEED[name], 16, K, N, residual=True)
+    A, Q = convert(tm, d, N, K)
+    W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], 128)
+    for T in (1, 4, 8, 16):
+        dd = dict(d, X=d["X"][:T], R=d["R"][:T])
+        want = O.epilogue(O.gemm_acc(dd["X"], W), kind, dd["R"] if kind == 2 else None)
+        got = run(tm, gemm, dd, A, Q, T, K, N, kind)
+        err = O.max_abs_rel(got, want)
+        assert err <= TOL, (name, T, err)
+
+
+@pytest.mark.parametrize("name,K,N,kind", LLAMA7B)
+def test_llama7b_prefill_shapes_sampled_rows(tm, gemm, name, K, N, kind):
+    # T = 2048 on the GPU; the oracle checks 96 of the 2048 token rows (first, last and random
+    # rows: output rows are independent, so this covers every column and every tile row class)
+    T = 2048
+    d = O.make_inputs(SEED[name] + 1, T, K, N, residual=True)
+    A, Q = convert(tm, d, N, K)
+    got = run(tm, gemm, d, A, Q, T, K, N, kind)
+    rng = np.random.default_rng(0)
+    rows = np.unique(np.concatenate([[0, 1, 15, 16, 255, 256, T - 1], rng.integers(0, T, 89)]))
+    W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], 128)
+    want = O.epilogue(O.gemm_acc(d["X"][rows], W), kind, d["R"][rows] if kind == 2 else None)
+    err = O.max_abs_rel(got[rows], want)
+    assert np.isfinite(got).all() and err <= TOL, (name, err)
+
+
+def test_errors(tm, gemm):
+    T, K, N = 4, 256, 64
+    d = O.make_inputs(1, T, K, N)
+    A, Q = convert(tm, d, N, K)
+    X = dev(d["X"])
+    C = torch.empty(T, N, dtype=torch.float16, device="cuda")
+    with pytest.raises(tm.W4A16Error, match="unsupported group size") as e:
+        gemm.Run(C, A, X, Q, N, T, K, 64)
+    assert e.value.code == -1
+    with pytest.raises(tm.W4A16Error, match="no feasible kernel found") as e:
+        gemm.Run(C, A, X, Q, N + 8, T, K, 128)
+    assert e.value.code == -2
+    with pytest.raises(tm.W4A16Error) as e:
+        gemm.Run(C, A, X, Q, N, T, K, 128, 0, 10 ** 6)
+    assert e.value.code == -5
+    with pytest.raises(tm.W4A16Error) as e:
+        gemm.Run(C, A, X, Q, N, T, K, 128, gemm.kFusedAdd)        # residual missing
+    assert e.value.code == -4
+    gemm.Run(C, A, X, Q, N, 0, K, 128)                            # zero tokens: no-op
+
+
+def test_measure_reports_all_kernels(tm, gemm):
+    T, K, N = 8, 1024, 256
+    d = O.make_inputs(2, T, K, N)
+    A, Q = convert(tm, d, N, K)
+    C = torch.empty(T, N, dtype=torch.float16, device="cuda")
+    ms = gemm.Measure(C, A, dev(d["X"]), Q, N, T, K, 128)
+    assert len(ms) == gemm.algo_count()
+    feas = [m for m in ms if m.feasible]
+    assert feas and all(np.isfinite(m.ms) and m.count == 100 for m in feas)
+    assert [m.ms for m in ms] == sorted(m.ms for m in ms)
+    assert sum(m.best for m in ms) == 1
