@@ -25,7 +25,7 @@ struct Metric {
     int                id;
     bool               feasible;
     bool               prefer;
-    std::array<int, 3> cta_shape;  // {features, tokens, K slices}
+    std::array<int, 3> cta_shape;  // {features, tokens, K slices per workgroup}
     int                kind;       // 0 decode kernel, 1 MFMA prefill kernel
     float              grid_size;
     int                best;

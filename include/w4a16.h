@@ -46,14 +46,16 @@ typedef struct w4a16_metric {
     int   kind;        /* 0 = decode (skinny) kernel, 1 = MFMA prefill kernel   */
     int   tile_n;      /* output features per workgroup                         */
     int   tile_t;      /* tokens per workgroup                                  */
-    int   slices;      /* K-slices (waves along K) per workgroup                */
+    int   slices;      /* decode: K slices (wave groups) per workgroup            */
     int   grid;        /* workgroups launched                                   */
     float ms;          /* total time of `count` launches, +inf if not feasible  */
     int   count;       /* number of timed launches                              */
 } w4a16_metric;
 
 /* GemmS4F16::GemmS4F16 / ~GemmS4F16 (gemm_s4_f16.h:19-21, gemm_s4_f16.cu:236-252).
- * The handle owns two events and nothing else; it binds to the current device. */
+ * The handle owns two events and a fixed 64 MiB scratch buffer for split-K partial sums
+ * (plus arrival counters); it binds to the current device.  GEMMs issued through one
+ * handle must be ordered on one stream at a time, because they share that scratch. */
 int  w4a16_create(w4a16_handle** out);
 void w4a16_destroy(w4a16_handle* h);
 

@@ -37,10 +37,16 @@ bool aligned16(const void* p)
 }  // namespace
 
 struct w4a16_handle {
-    hipEvent_t ev_start{};
-    hipEvent_t ev_end{};
-    int        device{};
+    hipEvent_t     ev_start{};
+    hipEvent_t     ev_end{};
+    int            device{};
+    w4a16::Scratch scratch{};
 };
+
+namespace {
+constexpr size_t kWorkspaceBytes = 64u << 20;  // split-K partial tiles
+constexpr int    kCounters       = 1 << 16;    // one per column block and token row block
+}  // namespace
 
 namespace w4a16 {
 
@@ -50,15 +56,18 @@ namespace {
 std::vector<Algo> build_table()
 {
     std::vector<Algo> t;
-    for (int r : {1, 2, 4})
-        for (int s : {1, 2, 4, 8, 16}) {
-            if (r == 4 && s == 16) continue;
-            t.push_back(Algo{0, 16 * r, 16, s, r});
-        }
+    const int rd[3][2]   = {{1, 8}, {1, 4}, {2, 4}};                                                 // r, depth
+    const int wnsk[9][2] = {{8, 1}, {8, 2}, {4, 1}, {4, 2}, {4, 4}, {2, 4}, {2, 8}, {1, 8}, {1, 16}};  // wn, sk
+    for (auto& a : rd)
+        for (auto& b : wnsk) t.push_back(Algo{0, 16 * a[0] * b[0], 16, b[1], 0, DecodeConfig{a[0], b[0], b[1], a[1], 0}});
+    // with K split across workgroups as well
+    t.push_back(Algo{0, 128, 16, 1, 0, DecodeConfig{1, 8, 1, 8, 2}});
+    t.push_back(Algo{0, 256, 16, 1, 0, DecodeConfig{2, 8, 1, 4, 2}});
+    t.push_back(Algo{0, 64, 16, 4, 0, DecodeConfig{1, 4, 4, 8, 2}});
     for (int v = 0; v < prefill_variants(); ++v) {
         int tn = 0, tt = 0;
         prefill_tile(v, tn, tt);
-        t.push_back(Algo{1, tn, tt, 1, v});
+        t.push_back(Algo{1, tn, tt, 1, v, DecodeConfig{}});
     }
     return t;
 }
@@ -84,28 +93,27 @@ const Algo& algo_at(int id)
 bool algo_feasible(int id, int N, int T, int K)
 {
     const Algo& a = algo_at(id);
-    return a.kind == 0 ? decode_feasible(a.param, a.slices, N, T, K) : prefill_feasible(a.param, N, T, K);
+    return a.kind == 0 ? decode_feasible(a.dc, N, T, K) : prefill_feasible(a.param, N, T, K);
 }
 
-int algo_grid(int id, int N, int T, int K)
+int algo_grid(int id, int N, int T, int K, const Scratch& sc)
 {
     const Algo& a = algo_at(id);
-    return a.kind == 0 ? decode_grid(a.param, a.slices, N, T, K) : prefill_grid(a.param, N, T, K);
+    return a.kind == 0 ? decode_grid(a.dc, N, T, K, sc.ws_bytes, sc.cnt_len) : prefill_grid(a.param, N, T, K);
 }
 
-hipError_t algo_launch(int id, const GemmArgs& g, hipStream_t st)
+hipError_t algo_launch(int id, const GemmArgs& g, const Scratch& sc, hipStream_t st)
 {
     const Algo& a = algo_at(id);
-    return a.kind == 0 ? decode_launch(a.param, a.slices, g, st) : prefill_launch(a.param, g, st);
+    return a.kind == 0 ? decode_launch(a.dc, g, sc.ws, sc.ws_bytes, sc.cnt, sc.cnt_len, st) :
+                         prefill_launch(a.param, g, st);
 }
 
-// Heuristic choice.  Few tokens: the decode kernel, with enough K slices that the chip holds
-// about eight waves per CU and each wave still owns two or more quantisation groups; two
-// column tiles per wave once more than eight tokens share the activations.  Many tokens: the
-// MFMA prefill kernel whose tile count wastes the least of the last wave of workgroups.
+// Heuristic choice (the counterpart of Estimate, gemm_s4_f16.cu:184-206).  Many tokens: the
+// MFMA prefill kernel whose tile count wastes the least of the last round of workgroups.
+// Few tokens: the decode kernel, see below.
 int algo_pick(int N, int T, int K)
 {
-    const int G = K / 128;
     if (T <= 0 || N <= 0 || K <= 0) return -1;
     int best = -1;
     if (T >= 64) {
@@ -113,12 +121,11 @@ int algo_pick(int N, int T, int K)
         for (int id = 0; id < algo_count(); ++id) {
             const Algo& a = algo_at(id);
             if (a.kind != 1 || !algo_feasible(id, N, T, K)) continue;
-            const double grid   = algo_grid(id, N, T, K);
+            const double grid   = prefill_grid(a.param, N, T, K);
             const double rounds = std::ceil(grid / 256.0);
             // time ~ rounds * work per tile, with a mild bonus for larger tiles (operand reuse)
             const double per_tile = (double)a.tile_n * a.tile_t;
-            const double padded_t = std::ceil((double)T / a.tile_t) * a.tile_t / T;
-            const double cost = rounds * per_tile * padded_t * (1.0 + 24.0 / a.tile_n + 24.0 / a.tile_t);
+            const double cost     = rounds * per_tile * (1.0 + 24.0 / a.tile_n + 24.0 / a.tile_t);
             if (cost < best_cost) {
                 best_cost = cost;
                 best      = id;
@@ -126,20 +133,29 @@ int algo_pick(int N, int T, int K)
         }
         if (best >= 0) return best;
     }
-    const int want_r = T > 8 && N % 32 == 0 ? 2 : 1;
-    for (int r = want_r; r >= 1 && best < 0; r >>= 1) {
-        const long tiles = (long)(N / (16 * r)) * ((T + 15) / 16);
-        int        s     = 16;
-        while (s > 1 && (tiles * s > 4096 || G / s < 2)) s >>= 1;
-        for (int id = 0; id < algo_count(); ++id) {
-            const Algo& a = algo_at(id);
-            if (a.kind == 0 && a.param == r && a.slices == s && algo_feasible(id, N, T, K)) {
-                best = id;
-                break;
-            }
-        }
+    // Decode: one column tile per wave, four groups in flight.  Wide matrices give every wave its
+    // own column tiles and share the activations among eight waves; narrow ones also slice K
+    // inside the workgroup so that at least 256 workgroups exist.  (From sweeps on MI355X.)
+    const int nt = N / 16;
+    int       wn, sk;
+    if (nt >= 1024) {
+        wn = 8, sk = 1;
     }
-    if (best >= 0) return best;
+    else if (nt >= 512) {
+        wn = 4, sk = 2;
+    }
+    else if (T <= 8) {
+        wn = 1, sk = 8;
+    }
+    else {
+        wn = 2, sk = 4;
+    }
+    for (int id = 0; id < algo_count(); ++id) {
+        const Algo& a = algo_at(id);
+        if (a.kind == 0 && a.dc.r == 1 && a.dc.depth == 4 && a.dc.wn == wn && a.dc.sk == sk && a.dc.fill == 0 &&
+            algo_feasible(id, N, T, K))
+            return id;
+    }
     for (int id = 0; id < algo_count(); ++id)
         if (algo_feasible(id, N, T, K)) return id;
     return -1;
@@ -180,11 +196,20 @@ int w4a16_create(w4a16_handle** out)
     hipError_t e = hipGetDevice(&h->device);
     if (e == hipSuccess) e = hipEventCreate(&h->ev_start);
     if (e == hipSuccess) e = hipEventCreate(&h->ev_end);
+    if (e == hipSuccess) e = hipMalloc((void**)&h->scratch.ws, kWorkspaceBytes);
+    if (e == hipSuccess) e = hipMalloc((void**)&h->scratch.cnt, kCounters * sizeof(int));
+    if (e == hipSuccess) e = hipMemset(h->scratch.cnt, 0, kCounters * sizeof(int));
+    if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
         if (h->ev_start) (void)hipEventDestroy(h->ev_start);
+        if (h->ev_end) (void)hipEventDestroy(h->ev_end);
+        if (h->scratch.ws) (void)hipFree(h->scratch.ws);
+        if (h->scratch.cnt) (void)hipFree(h->scratch.cnt);
         delete h;
         return hip_fail(e, "w4a16_create");
     }
+    h->scratch.ws_bytes = kWorkspaceBytes;
+    h->scratch.cnt_len  = kCounters;
     *out = h;
     return W4A16_OK;
 }
@@ -194,6 +219,8 @@ void w4a16_destroy(w4a16_handle* h)
     if (!h) return;
     (void)hipEventDestroy(h->ev_end);
     (void)hipEventDestroy(h->ev_start);
+    (void)hipFree(h->scratch.ws);
+    (void)hipFree(h->scratch.cnt);
     delete h;
 }
 
@@ -213,7 +240,7 @@ int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const voi
     if (algo_id < 0 || !algo_feasible(algo_id, n_out, tokens, k)) return fail(W4A16_ESHAPE, "no feasible kernel found");
     GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
                n_out,        tokens,             k,                  epilogue};
-    const hipError_t e = algo_launch(algo_id, g, (hipStream_t)stream);
+    const hipError_t e = algo_launch(algo_id, g, h->scratch, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "w4a16_gemm launch");
     return W4A16_OK;
 }
@@ -244,10 +271,10 @@ int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const 
         m.count    = 1;
         m.ms       = std::numeric_limits<float>::infinity();
         if (m.feasible) {
-            m.grid = algo_grid(id, n_out, tokens, k);
+            m.grid = algo_grid(id, n_out, tokens, k, h->scratch);
             for (int j = 0; j < kWarmup + kMeasure; ++j) {
                 if (j == kWarmup) (void)hipEventRecord(h->ev_start, st);
-                const hipError_t e = algo_launch(id, g, st);
+                const hipError_t e = algo_launch(id, g, h->scratch, st);
                 if (e != hipSuccess) return hip_fail(e, "w4a16_measure launch");
             }
             (void)hipEventRecord(h->ev_end, st);

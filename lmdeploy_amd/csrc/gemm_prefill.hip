@@ -47,7 +47,8 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     const int T0     = tile_t * TT;
     const int nt0    = (tile_n * TN) / kTileN + wave * NTW;  // first weight tile of this wave
 
-    const u32x4_t*  Ap = A + ((int64_t)nt0 * G) * 64 + lane;
+    const int64_t   gstride = (int64_t)(N / kTileN) * 64;  // 16-byte units between consecutive groups
+    const u32x4_t*  Ap      = A + (int64_t)nt0 * 64 + lane;  // + g * gstride + nt * 64
     const uint32_t* Qp = Q + nt0 * kTileN + c;
 
     // X staging: chunk (q*256 + tid) -> row q*16 + tid/16, 16-byte column tid%16
@@ -72,7 +73,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     uint32_t qv[NTW], qn[NTW];
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
-        w[nt]  = Ap[((int64_t)nt * G) * 64];
+        w[nt]  = Ap[nt * 64];
         qv[nt] = Qp[nt * kTileN];
     }
     // first activation tile
@@ -89,7 +90,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         if (more) {
 #pragma unroll
             for (int nt = 0; nt < NTW; ++nt) {
-                wn[nt] = Ap[((int64_t)nt * G + g + 1) * 64];
+                wn[nt] = Ap[(g + 1) * gstride + nt * 64];
                 qn[nt] = Qp[(int64_t)(g + 1) * N + nt * kTileN];
             }
         }

@@ -35,12 +35,12 @@ repack_weights_kernel(uint32_t* __restrict__ dst, const uint32_t* __restrict__ s
     const int64_t w     = global_id();
     const int64_t words = (int64_t)N * K / 8;
     if (w >= words) return;
-    const int     KT   = K / kGroup;
+    const int     NT   = N / kTileN;
     const int     j    = (int)(w & 3);
     const int     lane = (int)((w >> 2) & 63);
     const int64_t tile = w >> 8;
-    const int     nt   = (int)(tile / KT);
-    const int     kt   = (int)(tile % KT);
+    const int     kt   = (int)(tile / NT);
+    const int     nt   = (int)(tile % NT);
     const int     n    = nt * kTileN + (lane & 15);
     const int     k0   = kt * kGroup + 32 * j + 8 * (lane >> 4);
     const int     ld   = N / 8;
@@ -74,14 +74,14 @@ unrepack_weights_kernel(uint32_t* __restrict__ dst, const uint32_t* __restrict__
     const int ld = N / 8;
     const int k  = (int)(w / ld);
     const int n0 = (int)(w % ld) * 8;
-    const int KT = K / kGroup;
+    const int NT = N / kTileN;
     const int kt = k / kGroup, r = k % kGroup;
     const int j = r >> 5, b = (r >> 3) & 3, e = r & 7;
     uint32_t  out = 0;
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
         const int     n  = n0 + c;
-        const int64_t sw = (((int64_t)(n / kTileN) * KT + kt) * 64 + b * 16 + (n % kTileN)) * 4 + j;
+        const int64_t sw = (((int64_t)kt * NT + n / kTileN) * 64 + b * 16 + (n % kTileN)) * 4 + j;
         out |= nib(A[sw], nibble_of_row(e)) << (4 * nibble_of_row(c));
     }
     dst[w] = out;
@@ -111,12 +111,12 @@ dequantize_repacked_kernel(uint16_t* __restrict__ W, const uint32_t* __restrict_
     const int64_t w     = global_id();
     const int64_t words = (int64_t)N * K / 8;
     if (w >= words) return;
-    const int     KT   = K / kGroup;
+    const int     NT   = N / kTileN;
     const int     j    = (int)(w & 3);
     const int     lane = (int)((w >> 2) & 63);
     const int64_t tile = w >> 8;
-    const int     nt   = (int)(tile / KT);
-    const int     kt   = (int)(tile % KT);
+    const int     kt   = (int)(tile / NT);
+    const int     nt   = (int)(tile % NT);
     const int     n    = nt * kTileN + (lane & 15);
     const int     k0   = kt * kGroup + 32 * j + 8 * (lane >> 4);
     half2_t       z1024, z64;
@@ -204,12 +204,12 @@ from_reference_kernel(uint32_t* __restrict__ dst, const uint32_t* __restrict__ r
     const int64_t w     = global_id();
     const int64_t words = (int64_t)N * K / 8;
     if (w >= words) return;
-    const int     KT   = K / kGroup;
+    const int     NT   = N / kTileN;
     const int     j    = (int)(w & 3);
     const int     lane = (int)((w >> 2) & 63);
     const int64_t tile = w >> 8;
-    const int     nt   = (int)(tile / KT);
-    const int     kt   = (int)(tile % KT);
+    const int     kt   = (int)(tile / NT);
+    const int     nt   = (int)(tile % NT);
     const int     n    = nt * kTileN + (lane & 15);
     const int     k0   = kt * kGroup + 32 * j + 8 * (lane >> 4);
     uint32_t      out  = 0;

@@ -20,7 +20,10 @@ constexpr int kTileN = 16;   // columns of one weight tile
 constexpr int kWave  = 64;
 
 // Layout of the repacked weights.  One tile = 16 columns x 128 rows = 1024 bytes, stored as
-// 64 lanes x uint4.  Tile index = nt * (K/128) + kt.  Lane l = 16*b + c holds column
+// 64 lanes x uint4.  Tile index = kt * (N/16) + nt: the column tiles of one group are
+// contiguous, so waves on neighbouring columns stream neighbouring DRAM pages (measured: about
+// 10 % more bandwidth on a 240 MB matrix than with the tiles of a column contiguous).
+// Lane l = 16*b + c holds column
 // 16*nt + c; its word j holds rows 128*kt + 32*j + 8*b + e (e = 0..7), row offset e in
 // nibble kNibbleOfRow[e].  One word is therefore one B operand of v_mfma_f32_16x16x32_f16.
 // Pack order along the rows is the AWQ order [0,2,4,6,1,3,5,7], which lets the unpack

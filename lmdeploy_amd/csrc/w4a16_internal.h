@@ -19,12 +19,28 @@ struct GemmArgs {
 };
 
 // One dispatchable kernel configuration.
+// A decode kernel configuration: r column tiles per wave, wn waves per slice, sk slices per
+// workgroup, `depth` groups of weights in flight per wave; fill > 0 additionally splits K
+// across workgroups until about `fill` workgroups per CU exist.
+struct DecodeConfig {
+    int r, wn, sk, depth, fill;
+};
+
 struct Algo {
-    int kind;     // 0 decode, 1 prefill
-    int tile_n;   // output features per workgroup
-    int tile_t;   // tokens per workgroup
-    int slices;   // waves along K per workgroup (decode) / 1
-    int param;    // kernel-specific variant index
+    int          kind;     // 0 decode, 1 prefill
+    int          tile_n;   // output features per workgroup
+    int          tile_t;   // tokens per workgroup
+    int          slices;   // K slices per workgroup
+    int          param;    // prefill: variant index
+    DecodeConfig dc;       // decode only
+};
+
+// Scratch owned by a handle: split-K partial tiles and arrival counters.
+struct Scratch {
+    float* ws;
+    size_t ws_bytes;
+    int*   cnt;
+    int    cnt_len;
 };
 
 int         algo_count();
@@ -34,8 +50,8 @@ bool algo_feasible(int id, int N, int T, int K);
 // heuristic choice (the counterpart of Estimate); -1 if nothing is feasible
 int algo_pick(int N, int T, int K);
 // workgroups the launch would use
-int algo_grid(int id, int N, int T, int K);
-hipError_t algo_launch(int id, const GemmArgs& a, hipStream_t st);
+int algo_grid(int id, int N, int T, int K, const Scratch& sc);
+hipError_t algo_launch(int id, const GemmArgs& a, const Scratch& sc, hipStream_t st);
 
 hipError_t launch_convert(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* A_src, const uint16_t* scales,
                           const uint32_t* qzeros, int m, int k, hipStream_t st);
@@ -48,10 +64,11 @@ hipError_t launch_fuse_w1_w3(uint32_t* dst, const uint32_t* src, int m, int k, h
 hipError_t launch_transpose_qk(uint32_t* dst, const uint32_t* src, int m, int k, int size_per_head, hipStream_t st);
 hipError_t launch_from_reference(uint32_t* dst, const uint32_t* ref, int m, int k, hipStream_t st);
 
-// decode (skinny) kernels: R column tiles per wave x S waves along K
-bool       decode_feasible(int r, int s, int N, int T, int K);
-int        decode_grid(int r, int s, int N, int T, int K);
-hipError_t decode_launch(int r, int s, const GemmArgs& a, hipStream_t st);
+// decode (skinny) kernels
+bool       decode_feasible(const DecodeConfig& cf, int N, int T, int K);
+int        decode_grid(const DecodeConfig& cf, int N, int T, int K, size_t ws_bytes, int cnt_len);
+hipError_t decode_launch(const DecodeConfig& cf, const GemmArgs& a, float* ws, size_t ws_bytes, int* cnt, int cnt_len,
+                         hipStream_t st);
 
 // MFMA prefill kernels
 int        prefill_variants();

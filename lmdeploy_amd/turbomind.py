@@ -105,7 +105,7 @@ class GemmS4F16:
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
-        if h:
+        if h and lib is not None:  # `lib` is already gone at interpreter shutdown
             lib.w4a16_destroy(h)
 
     def Run(self, C, A, B, Q, m: int, n: int, k: int, group_size: int, type: int = 0, algo_id: int = -1,

@@ -296,7 +296,9 @@ def max_abs_rel(y: np.ndarray, yref: np.ndarray) -> float:
 # The gfx950 tiled layout produced by this build's convert_s4_k_m8 (specification).
 # ---------------------------------------------------------------------------
 # Weights: one tile = 16 columns x 128 rows (one quantisation group) = 1024 bytes, stored as
-# 64 lanes x one 16-byte vector.  Tile index = nt * (K/128) + kt.  Lane l = 16*b + c holds
+# 64 lanes x one 16-byte vector.  Tile index = kt * (N/16) + nt (all column tiles of a group
+# are contiguous, so that waves working on neighbouring columns read neighbouring DRAM
+# pages).  Lane l = 16*b + c holds
 # column n = 16*nt + c; its word j (0..3) holds rows k = 128*kt + 32*j + 8*b + e, e = 0..7,
 # with row offset e in nibble p where e = AWQ_ORDER[p].  That is exactly one operand of
 # v_mfma_f32_16x16x32_f16 per word, and the in-register unpack needs a single shift.
@@ -305,11 +307,11 @@ TILE_N, TILE_K = 16, 128
 
 def gfx950_layout_element(N: int, K: int, word_index: int, nib: int):
     """(k, n) held by nibble `nib` of word `word_index` of the repacked weight buffer."""
-    KT = K // TILE_K
+    NT = N // TILE_N
     j = word_index & 3
     lane = (word_index >> 2) & 63
     tile = word_index >> 8
-    nt, kt = divmod(tile, KT)
+    kt, nt = divmod(tile, NT)
     c, b = lane & 15, lane >> 4
     return TILE_K * kt + 32 * j + 8 * b + AWQ_ORDER[nib], TILE_N * nt + c
 
@@ -321,7 +323,7 @@ def repack_gfx950(qweight: np.ndarray, N: int, K: int) -> np.ndarray:
     NT, KT = N // TILE_N, K // TILE_K
     # k = 128 kt + 32 j + 8 b + e ; n = 16 nt + c
     t = q.reshape(KT, 4, 4, 8, NT, 16)                         # kt, j, b, e, nt, c
-    t = t.transpose(4, 0, 2, 5, 1, 3)                          # nt, kt, b, c, j, e
+    t = t.transpose(0, 4, 2, 5, 1, 3)                          # kt, nt, b, c, j, e
     nib = t[..., list(AWQ_ORDER)]                              # nibble p <- e = AWQ_ORDER[p]
     return nibbles_to_words(np.ascontiguousarray(nib)).reshape(-1)
 
@@ -329,10 +331,10 @@ def repack_gfx950(qweight: np.ndarray, N: int, K: int) -> np.ndarray:
 def unrepack_gfx950(A: np.ndarray, N: int, K: int) -> np.ndarray:
     """Inverse of repack_gfx950: tiled words -> logical q uint8 [K, N]."""
     NT, KT = N // TILE_N, K // TILE_K
-    nib = words_to_nibbles(np.asarray(A, dtype=np.uint32).reshape(NT, KT, 4, 16, 4))
+    nib = words_to_nibbles(np.asarray(A, dtype=np.uint32).reshape(KT, NT, 4, 16, 4))
     e = np.empty_like(nib)
     e[..., list(AWQ_ORDER)] = nib                              # e index <- nibble p
-    t = e.transpose(1, 4, 2, 5, 0, 3)                          # kt, j, b, e, nt, c
+    t = e.transpose(0, 4, 2, 5, 1, 3)                          # kt, j, b, e, nt, c
     return np.ascontiguousarray(t).reshape(K, N)
 
 
