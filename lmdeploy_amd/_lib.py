@@ -7,7 +7,8 @@ import os
 from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libw4a16.so")
+# W4A16_LIB overrides the in-tree library (e.g. to try a differently tuned build)
+LIB_PATH = os.environ.get("W4A16_LIB") or os.path.join(_HERE, "lib", "libw4a16.so")
 
 OK, EGROUP, ESHAPE, EHIP, EARG, EALGO = 0, -1, -2, -3, -4, -5
 GEMM, FUSED_SILU_FFN, FUSED_ADD = 0, 1, 2

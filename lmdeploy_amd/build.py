@@ -29,15 +29,36 @@ def _hipcc() -> str:
     return exe
 
 
+# The GEMM kernels wait for their software-pipelined loads by count.  A register spill would put
+# scratch stores among those loads, and stores complete out of order with loads, so a spilling
+# GEMM kernel is a wrong kernel: the build refuses it.
+NO_SCRATCH = ("gemm_decode.hip", "gemm_prefill.hip")
+
+
+def _check_no_scratch(src: str, remarks: str) -> None:
+    name = None
+    for line in remarks.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in line:
+            size = int(line.split("ScratchSize [bytes/lane]:")[1].split("[")[0])
+            if size != 0:
+                raise RuntimeError("%s: kernel %s spills %d bytes/lane to scratch" % (src, name, size))
+
+
 def _compile(src: str, obj_dir: str) -> str:
     obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
     cmd = [_hipcc(), *HIP_FLAGS]
     if src.endswith(".cpp"):
         cmd += ["-x", "hip"]
+    if src in NO_SCRATCH:
+        cmd += ["-Rpass-analysis=kernel-resource-usage"]
     cmd += ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
+    if src in NO_SCRATCH:
+        _check_no_scratch(src, r.stderr)
     return obj
 
 

@@ -61,9 +61,11 @@ std::vector<Algo> build_table()
     for (auto& a : rd)
         for (auto& b : wnsk) t.push_back(Algo{0, 16 * a[0] * b[0], 16, b[1], 0, DecodeConfig{a[0], b[0], b[1], a[1], 0}});
     // with K split across workgroups as well
-    t.push_back(Algo{0, 128, 16, 1, 0, DecodeConfig{1, 8, 1, 8, 2}});
-    t.push_back(Algo{0, 256, 16, 1, 0, DecodeConfig{2, 8, 1, 4, 2}});
-    t.push_back(Algo{0, 64, 16, 4, 0, DecodeConfig{1, 4, 4, 8, 2}});
+    for (int fill : {1, 2, 4}) {
+        t.push_back(Algo{0, 128, 16, 1, 0, DecodeConfig{1, 8, 1, 4, fill}});
+        t.push_back(Algo{0, 64, 16, 1, 0, DecodeConfig{1, 4, 1, 4, fill}});
+        t.push_back(Algo{0, 128, 16, 2, 0, DecodeConfig{1, 8, 2, 4, fill}});
+    }
     for (int v = 0; v < prefill_variants(); ++v) {
         int tn = 0, tt = 0;
         prefill_tile(v, tn, tt);
@@ -115,44 +117,42 @@ hipError_t algo_launch(int id, const GemmArgs& g, const Scratch& sc, hipStream_t
 int algo_pick(int N, int T, int K)
 {
     if (T <= 0 || N <= 0 || K <= 0) return -1;
-    int best = -1;
     if (T >= 64) {
-        double best_cost = std::numeric_limits<double>::infinity();
-        for (int id = 0; id < algo_count(); ++id) {
-            const Algo& a = algo_at(id);
-            if (a.kind != 1 || !algo_feasible(id, N, T, K)) continue;
-            const double grid   = prefill_grid(a.param, N, T, K);
-            const double rounds = std::ceil(grid / 256.0);
-            // time ~ rounds * work per tile, with a mild bonus for larger tiles (operand reuse)
-            const double per_tile = (double)a.tile_n * a.tile_t;
-            const double cost     = rounds * per_tile * (1.0 + 24.0 / a.tile_n + 24.0 / a.tile_t);
-            if (cost < best_cost) {
-                best_cost = cost;
-                best      = id;
+        // 128 x 128 tiles (two workgroups per CU hide each other's memory latency) were the
+        // fastest on every Llama shape measured; narrower token tiles for short prompts.
+        const int order[5][2] = {{128, 128}, {64, 128}, {64, 64}, {128, 256}, {256, 128}};  // tokens, features
+        for (auto& o : order) {
+            if (T <= 64 && o[0] > 64) continue;
+            for (int id = 0; id < algo_count(); ++id) {
+                const Algo& a = algo_at(id);
+                if (a.kind == 1 && a.tile_t == o[0] && a.tile_n == o[1] && algo_feasible(id, N, T, K)) return id;
             }
         }
-        if (best >= 0) return best;
+        for (int id = 0; id < algo_count(); ++id)
+            if (algo_at(id).kind == 1 && algo_feasible(id, N, T, K)) return id;
     }
     // Decode: one column tile per wave, four groups in flight.  Wide matrices give every wave its
     // own column tiles and share the activations among eight waves; narrow ones also slice K
     // inside the workgroup so that at least 256 workgroups exist.  (From sweeps on MI355X.)
-    const int nt = N / 16;
-    int       wn, sk;
+    const int nt = N / 16, groups = K / 128;
+    int       wn, sk, fill = 0;
     if (nt >= 1024) {
         wn = 8, sk = 1;
     }
     else if (nt >= 512) {
         wn = 4, sk = 2;
     }
-    else if (T <= 8) {
-        wn = 1, sk = 8;
+    else if (T > 8 || (T > 4 && groups >= 64)) {
+        // narrow matrix, many tokens: the activations dominate the traffic unless eight waves
+        // share them, so K is split across workgroups instead of inside them
+        wn = 8, sk = 1, fill = 1;
     }
     else {
-        wn = 2, sk = 4;
+        wn = 1, sk = 8;
     }
     for (int id = 0; id < algo_count(); ++id) {
         const Algo& a = algo_at(id);
-        if (a.kind == 0 && a.dc.r == 1 && a.dc.depth == 4 && a.dc.wn == wn && a.dc.sk == sk && a.dc.fill == 0 &&
+        if (a.kind == 0 && a.dc.r == 1 && a.dc.depth == 4 && a.dc.wn == wn && a.dc.sk == sk && a.dc.fill == fill &&
             algo_feasible(id, N, T, K))
             return id;
     }

@@ -32,7 +32,7 @@ namespace w4a16 {
 namespace {
 
 constexpr int    kMaxWaves = 16;
-constexpr size_t kMaxLds   = 64 * 1024;
+constexpr size_t kMaxLds   = 128 * 1024;  // of the CU's 160 KiB; more than 64 KiB needs an opt-in per kernel
 
 template<int R>
 struct Stage {
@@ -308,15 +308,27 @@ decode_kernel(const DecodeParams p)
         }
         __syncthreads();
         if (!last_flag || slice != 0) return;
+        // sum the SK partials in split order; eight splits' loads are in flight at a time (a
+        // load-add-load-add chain would pay one memory round trip per split)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             acc[r] = float4_t{0.f, 0.f, 0.f, 0.f};
-            for (int s = 0; s < p.SK; ++s) {
-                const float* wp = p.ws + ((zs + s) * NT + nt[r]) * 256 + lane;
+            for (int s0 = 0; s0 < p.SK; s0 += 8) {
+                float v[8][4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (4 * b + i < Tl)
-                        acc[r][i] += __hip_atomic_load(wp + i * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int u = 0; u < 8; ++u) {
+                    const float* wp = p.ws + ((zs + min(s0 + u, p.SK - 1)) * NT + nt[r]) * 256 + lane;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        v[u][i] = __hip_atomic_load(wp + i * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (s0 + u < p.SK) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) acc[r][i] += v[u][i];
+                    }
+                }
             }
         }
     }
@@ -357,11 +369,26 @@ decode_kernel(const DecodeParams p)
 template<int R, int TP, int D>
 hipError_t launch_rtd(const DecodeParams& p, dim3 grid, dim3 block, size_t lds, int epilogue, hipStream_t st)
 {
+#define W4A16_LAUNCH(EPI)                                                                                              \
+    do {                                                                                                               \
+        auto kfn = decode_kernel<R, TP, D, EPI>;                                                                       \
+        if (lds > 64 * 1024) {                                                                                         \
+            static bool raised = false; /* per instantiation */                                                       \
+            if (!raised) {                                                                                             \
+                const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),                           \
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);    \
+                if (e != hipSuccess) return e;                                                                         \
+                raised = true;                                                                                         \
+            }                                                                                                          \
+        }                                                                                                              \
+        hipLaunchKernelGGL(kfn, grid, block, lds, st, p);                                                              \
+    } while (0)
     switch (epilogue) {
-        case kEpiGemm: hipLaunchKernelGGL((decode_kernel<R, TP, D, kEpiGemm>), grid, block, lds, st, p); break;
-        case kEpiSilu: hipLaunchKernelGGL((decode_kernel<R, TP, D, kEpiSilu>), grid, block, lds, st, p); break;
-        default: hipLaunchKernelGGL((decode_kernel<R, TP, D, kEpiAdd>), grid, block, lds, st, p); break;
+        case kEpiGemm: W4A16_LAUNCH(kEpiGemm); break;
+        case kEpiSilu: W4A16_LAUNCH(kEpiSilu); break;
+        default: W4A16_LAUNCH(kEpiAdd); break;
     }
+#undef W4A16_LAUNCH
     return hipGetLastError();
 }
 

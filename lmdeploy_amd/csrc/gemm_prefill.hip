@@ -13,29 +13,70 @@
 #include "w4a16_common.h"
 #include "w4a16_internal.h"
 
+#include <type_traits>
+
 namespace w4a16 {
 
 namespace {
 
 constexpr int kThreads   = 256;
-constexpr int kRowHalves = kGroup + 8;  // LDS row stride: 272 bytes, keeps 16 rows on distinct banks
+#ifndef W4A16_ROWPAD
+#define W4A16_ROWPAD 16
+#endif
+constexpr int kRowHalves = kGroup + W4A16_ROWPAD;  // LDS row stride 288 bytes: measured free of bank conflicts (272 is not)
 
+// Compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(<N-1>); gives inline assembly
+// its immediate operands.
+template<int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// Loads of the software pipeline.  They are issued from inline assembly, in place ("+v"), with
+// a scalar base and a per-thread 32-bit offset, and waited for by count: the compiler would
+// drain every load in flight at the loop header, exposing the memory latency once per K step.
+template<int OFF>
+__device__ __forceinline__ void gload128(u32x4_t& dst, uint32_t voff, const void* sbase)
+{
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "+v"(dst) : "v"(voff), "s"(sbase), "n"(OFF));
+}
+template<int OFF>
+__device__ __forceinline__ void gload32(uint32_t& dst, uint32_t voff, const void* sbase)
+{
+    asm volatile("global_load_dword %0, %1, %2 offset:%3" : "+v"(dst) : "v"(voff), "s"(sbase), "n"(OFF));
+}
+// wait until at most N of this wave's loads are in flight; tied to `v` so that no use of it can
+// be scheduled above the wait
+template<int N, typename V>
+__device__ __forceinline__ void wait_vm(V& v)
+{
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(v) : "n"(N));
+}
+
+// Register budget: one wave per SIMD (512 registers) for the 256-register accumulator tiles,
+// two waves otherwise.  Stating it keeps the allocator from squeezing the kernel into fewer
+// VGPRs and shuttling values through AGPRs inside the loop.
 template<int TTILES, int NTW, int EPI>
 __global__ void __launch_bounds__(kThreads)
+    __attribute__((amdgpu_waves_per_eu(TTILES * NTW >= 32 ? 1 : 2, TTILES * NTW >= 32 ? 1 : 2)))
 prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const uint16_t* __restrict__ X,
                const uint32_t* __restrict__ Q, const uint16_t* R_, int N, int T, int K, int tiles_t, int tiles_n)
 {
     extern __shared__ __attribute__((aligned(16))) uint16_t xs[];  // [2][TT][kRowHalves]
-    constexpr int TT   = 16 * TTILES;
-    constexpr int TN   = 64 * NTW;
-    constexpr int XPER = TTILES / 4;  // 16-byte chunks of X per thread and 32-wide K step
+    constexpr int TT = 16 * TTILES;
+    constexpr int TN = 64 * NTW;
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c    = lane & 15;
     const int b    = lane >> 4;
     const int G    = K / kGroup;
+    const int NT   = N / kTileN;
 
     // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous block of
     // tiles (all token tiles of a few feature tiles) so its private L2 sees the reuse.
@@ -47,17 +88,16 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     const int T0     = tile_t * TT;
     const int nt0    = (tile_n * TN) / kTileN + wave * NTW;  // first weight tile of this wave
 
-    const int64_t   gstride = (int64_t)(N / kTileN) * 64;  // 16-byte units between consecutive groups
-    const u32x4_t*  Ap      = A + (int64_t)nt0 * 64 + lane;  // + g * gstride + nt * 64
-    const uint32_t* Qp = Q + nt0 * kTileN + c;
-
-    // X staging: chunk (q*256 + tid) -> row q*16 + tid/16, 16-byte column tid%16
+    // per-thread byte offsets; the group-dependent part of every address is scalar
+    const uint32_t w_off = (uint32_t)(nt0 * 1024 + lane * 16);        // + g * NT * 1024 (+ nt * 1024)
+    const uint32_t q_off = (uint32_t)((nt0 * kTileN + c) * 4);        // + g * N * 4    (+ nt * 64)
+    // X staging: chunk q of this thread is row q*16 + tid/16, 16-byte column tid%16 of the tile
     // (rows past the last token re-read the last valid row; their outputs are never stored)
-    const int  xr = tid >> 4, xc = tid & 15;
-    const auto x_chunk = [&](int q, int g) {
-        const int row = min(T0 + q * 16 + xr, T - 1);
-        return *reinterpret_cast<const u32x4_t*>(X + (int64_t)row * K + xc * 8 + g * kGroup);
-    };
+    const int xr = tid >> 4, xc = tid & 15;
+    uint32_t  x_off[TTILES];
+#pragma unroll
+    for (int q = 0; q < TTILES; ++q)
+        x_off[q] = (uint32_t)(min(T0 + q * 16 + xr, T - 1)) * (uint32_t)(K * 2) + xc * 16;  // + g * 256
     const int xs_w = xr * kRowHalves + xc * 8;  // + q*16*kRowHalves
     const int xs_r = c * kRowHalves + 8 * b;    // + tt*16*kRowHalves + 32*j
 
@@ -69,31 +109,59 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) acc[tt][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    u32x4_t  w[NTW], wn[NTW];
-    uint32_t qv[NTW], qn[NTW];
+    u32x4_t  wa[NTW], wb[NTW];  // weights of the current / next group (roles alternate)
+    uint32_t qa[NTW], qb[NTW];
+    constexpr int XB = TTILES < 8 ? TTILES : 8;  // activation chunks staged at a time
+    u32x4_t       xst[XB];                        // activations of the next group on their way to LDS
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
-        w[nt]  = Ap[nt * 64];
-        qv[nt] = Qp[nt * kTileN];
+        wa[nt] = wb[nt] = u32x4_t{0, 0, 0, 0};
+        qa[nt] = qb[nt] = 0;
     }
-    // first activation tile
 #pragma unroll
-    for (int q = 0; q < TTILES; ++q) {
-        const u32x4_t v = x_chunk(q, 0);
-        *reinterpret_cast<u32x4_t*>(&xs[xs_w + q * 16 * kRowHalves]) = v;
+    for (int q = 0; q < XB; ++q) xst[q] = u32x4_t{0, 0, 0, 0};
+
+    auto issue_w = [&](u32x4_t (&w)[NTW], uint32_t (&qv)[NTW], int g) {
+        const char* wbase = reinterpret_cast<const char*>(A) + (int64_t)g * NT * 1024;
+        const char* qbase = reinterpret_cast<const char*>(Q) + (int64_t)g * N * 4;
+        static_for<0, NTW>([&](auto nt) { gload128<nt * 1024>(w[nt], w_off, wbase); });
+        static_for<0, NTW>([&](auto nt) { gload32<nt * 64>(qv[nt], q_off, qbase); });
+    };
+    // activation chunks [q0, q0 + XB) of group g: request, and (later) wait for all and store
+    auto issue_x = [&](int q0, int g) {
+        const char* xbase = reinterpret_cast<const char*>(X) + (int64_t)g * 256;
+#pragma unroll
+        for (int q = 0; q < XB; ++q) gload128<0>(xst[q], x_off[q0 + q], xbase);
+    };
+    auto store_x = [&](uint16_t* xo, int q0) {
+#pragma unroll
+        for (int q = 0; q < XB; ++q) {
+            wait_vm<0>(xst[q]);
+            *reinterpret_cast<u32x4_t*>(&xo[xs_w + (q0 + q) * 16 * kRowHalves]) = xst[q];
+        }
+    };
+
+    // ---- prologue: group 0 ----
+    issue_w(wa, qa, 0);
+#pragma unroll
+    for (int q0 = 0; q0 < TTILES; q0 += XB) {
+        issue_x(q0, 0);
+        store_x(xs, q0);
+    }
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt) {
+        wait_vm<0>(wa[nt]);
+        wait_vm<0>(qa[nt]);
     }
     __syncthreads();
 
-    int buf = 0;
-    for (int g = 0; g < G; ++g) {
-        const bool more = g + 1 < G;
-        if (more) {
-#pragma unroll
-            for (int nt = 0; nt < NTW; ++nt) {
-                wn[nt] = Ap[(g + 1) * gstride + nt * 64];
-                qn[nt] = Qp[(int64_t)(g + 1) * N + nt * kTileN];
-            }
-        }
+    // One K step (a quantisation group): MFMAs on `w`/buffer `xb` while the next group's
+    // weights go to `wn` and its activations to the other LDS buffer `xo`.
+    auto step = [&](u32x4_t (&w)[NTW], uint32_t (&qv)[NTW], u32x4_t (&wn)[NTW], uint32_t (&qn)[NTW],
+                    const uint16_t* xb, uint16_t* xo, int g) {
+        const int gn = min(g + 1, G - 1);  // (the last step re-reads its own group: no branch)
+        issue_w(wn, qn, gn);
+        issue_x(0, gn);
         half2_t z1024[NTW], z64[NTW], sc[NTW];
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) {
@@ -101,41 +169,42 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
             split_q(qv[nt], z1024[nt], z64[nt], s);
             sc[nt] = half2_t{s, s};
         }
-        const uint16_t* xb = xs + buf * (TT * kRowHalves);
-        uint16_t*       xo = xs + (buf ^ 1) * (TT * kRowHalves);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            u32x4_t stage[XPER];
-            if (more) {
-#pragma unroll
-                for (int q = 0; q < XPER; ++q)
-                    stage[q] = x_chunk(j * XPER + q, g + 1);
-            }
-            half8_t wf[NTW];
+        static_for<0, 4>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            half8_t       wf[NTW];
 #pragma unroll
             for (int nt = 0; nt < NTW; ++nt) wf[nt] = dequant_full(w[nt][j], z1024[nt], z64[nt], sc[nt], uc);
 #pragma unroll
             for (int tt = 0; tt < TTILES; ++tt) {
-                const half8_t xf =
-                    *reinterpret_cast<const half8_t*>(&xb[xs_r + tt * 16 * kRowHalves + 32 * j]);
+                const half8_t xf = *reinterpret_cast<const half8_t*>(&xb[xs_r + tt * 16 * kRowHalves + 32 * j]);
 #pragma unroll
                 for (int nt = 0; nt < NTW; ++nt)
                     acc[tt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[nt], xf, acc[tt][nt], 0, 0, 0);
             }
-            if (more) {
-#pragma unroll
-                for (int q = 0; q < XPER; ++q)
-                    *reinterpret_cast<u32x4_t*>(&xo[xs_w + (j * XPER + q) * 16 * kRowHalves]) = stage[q];
+            // staged activations: with 16 token tiles the first 8 chunks are stored (and the other
+            // 8 requested) after the second k32 step; the last batch is stored after the fourth
+            if constexpr (TTILES > XB && j == 1) {
+                store_x(xo, 0);
+                issue_x(XB, gn);
             }
+            if constexpr (j == 3) store_x(xo, TTILES - XB);
+        });
+#pragma unroll
+        for (int nt = 0; nt < NTW; ++nt) {  // everything has landed (vmcnt(0) above); pin the uses below it
+            wait_vm<0>(wn[nt]);
+            wait_vm<0>(qn[nt]);
         }
         __syncthreads();
-        buf ^= 1;
-#pragma unroll
-        for (int nt = 0; nt < NTW; ++nt) {
-            w[nt]  = wn[nt];
-            qv[nt] = qn[nt];
-        }
+    };
+
+    uint16_t* const x0 = xs;
+    uint16_t* const x1 = xs + TT * kRowHalves;
+    int g = 0;
+    for (; g + 1 < G; g += 2) {  // no branch inside: the 4*TTILES*NTW accumulators stay in place
+        step(wa, qa, wb, qb, x0, x1, g);
+        step(wb, qb, wa, qa, x1, x0, g + 1);
     }
+    if (g < G) step(wa, qa, wb, qb, x0, x1, g);
 
     // ---- epilogue: lane (c, b) of tile (tt, nt) holds token T0 + 16 tt + c, features n .. n+3 ----
 #pragma unroll
@@ -174,7 +243,9 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
 struct Variant {
     int ttiles, ntw;
 };
-constexpr Variant kVariants[] = {{16, 4}, {8, 4}, {16, 2}, {8, 2}, {4, 2}, {4, 1}};
+// (a 256 x 256 tile does not fit the register file without spilling, and spill stores would
+// break the counted waits: stores and loads complete out of order with each other)
+constexpr Variant kVariants[] = {{8, 4}, {16, 2}, {8, 2}, {4, 2}, {4, 1}};
 constexpr int     kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 template<int TTILES, int NTW>
@@ -221,6 +292,8 @@ bool prefill_feasible(int v, int N, int T, int K)
     if (v < 0 || v >= kNumVariants || N <= 0 || T <= 0 || K <= 0) return false;
     const int tn = 64 * kVariants[v].ntw, tt = 16 * kVariants[v].ttiles;
     if (N % tn != 0 || K % kGroup != 0) return false;
+    // per-thread offsets into X and into one group of A are 32-bit
+    if ((int64_t)T * K * 2 >= (1ll << 32) || (int64_t)N * 64 >= (1ll << 32)) return false;
     const int64_t grid = (int64_t)(N / tn) * ((T + tt - 1) / tt);
     return grid < (1ll << 31);
 }
@@ -235,11 +308,10 @@ int prefill_grid(int v, int N, int T, int K)
 hipError_t prefill_launch(int v, const GemmArgs& a, hipStream_t st)
 {
     switch (v) {
-        case 0: return launch_v<16, 4>(a, st);
-        case 1: return launch_v<8, 4>(a, st);
-        case 2: return launch_v<16, 2>(a, st);
-        case 3: return launch_v<8, 2>(a, st);
-        case 4: return launch_v<4, 2>(a, st);
+        case 0: return launch_v<8, 4>(a, st);
+        case 1: return launch_v<16, 2>(a, st);
+        case 2: return launch_v<8, 2>(a, st);
+        case 3: return launch_v<4, 2>(a, st);
         default: return launch_v<4, 1>(a, st);
     }
 }
