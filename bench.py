@@ -28,6 +28,12 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16 matrix
 
+# HBM bytes per launch of the two dominant kernels, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
+# runs of `bench.py --probe ...`, calibrated against an elementwise kernel of known size
+# (profiles/decode_gate_up_hbm_traffic.md, profiles/prefill_gate_up_mfma_and_traffic.md).
+TRAFFIC_DECODE_GATE_UP = 48.66e6
+TRAFFIC_PREFILL_GATE_UP = 558.7e6
+
 # name, K, N (gate_up: both halves), epilogue
 LAYER_7B = [("qkv", 4096, 12288, 0), ("o", 4096, 4096, 0), ("gate_up", 4096, 22016, 1), ("down", 11008, 4096, 2)]
 DECODE_T = (1, 4, 8, 16)
@@ -78,6 +84,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-per-shape", action="store_true")
+    ap.add_argument("--probe", choices=["decode", "prefill"],
+                    help="run only the dominant kernel of that regime plus a plain 256 MiB device copy, "
+                         "eagerly, for `rocprofv3 --pmc` (no JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -139,6 +148,22 @@ def main():
             torch.cuda.synchronize()
         return e0.elapsed_time(e1)   # ms
 
+    if args.probe:
+        # a plain copy of known size calibrates FETCH_SIZE / WRITE_SIZE, then the kernel on cold weights
+        src = torch.zeros(64 * 2 ** 20, dtype=torch.int32, device="cuda")   # 256 MiB
+        dst = torch.empty_like(src)
+        with torch.cuda.stream(stream):
+            for _ in range(4):
+                torch.add(src, 1, out=dst)   # an elementwise kernel: reads 256 MiB, writes 256 MiB
+            n = len(weights["gate_up"])
+            for rep in range(2):
+                for c in range(n):
+                    launch("gate_up", c, DECODE_T[c % len(DECODE_T)] if args.probe == "decode" else PREFILL_T,
+                           stream.cuda_stream)
+        torch.cuda.synchronize()
+        print("probe done: 4 add kernels over 268435456 bytes, %d gate_up launches (%s)" % (2 * n, args.probe))
+        return
+
     # ---- headline: the decode layer set, one layer copy per step ------------------------------
     step_bytes = sum(algorithmic_bytes(T, K, N, epi) for T in DECODE_T for _, K, N, epi in LAYER_7B)
     runner = make_runner([[(name, c, T) for T in DECODE_T for name, _, _, _ in LAYER_7B] for c in range(args.copies)])
@@ -158,7 +183,7 @@ def main():
     gu_us = per_launch_us("gate_up", DECODE_T, passes=6)
     achieved = gu_bytes / (gu_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_DECODE_GATE_UP,
                 "kernel": "decode_kernel, gate_up K=4096 N=22016 +SiLU, T cycling over {1,4,8,16}",
                 "bytes_per_launch": int(gu_bytes), "us_per_launch": round(gu_us, 3)}
 
@@ -188,7 +213,8 @@ def main():
         prefill = {"T": PREFILL_T, "TFLOPs": round(tot_fl / tot_ms / 1e9, 1), "ms_per_layer": round(tot_ms, 4),
                    "per_shape": rows,
                    "roofline": {"bound": "mfma", "achieved": dom["TFLOPs"], "peak": MFMA_PEAK_TFLOPS,
-                                "unit": "TFLOP/s", "frac": dom["frac"], "traffic": None,
+                                "unit": "TFLOP/s", "frac": dom["frac"],
+                                "traffic": TRAFFIC_PREFILL_GATE_UP if dom["shape"] == "gate_up" else None,
                                 "kernel": "prefill_kernel, %s, T=2048" % dom["shape"]}}
 
     # ---- CPU baseline: the oracle on the host cores, one layer at T = 8 -------------------------

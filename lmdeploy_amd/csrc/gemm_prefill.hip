@@ -78,13 +78,24 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     const int G    = K / kGroup;
     const int NT   = N / kTileN;
 
-    // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous block of
-    // tiles (all token tiles of a few feature tiles) so its private L2 sees the reuse.
+    // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of tiles so
+    // its private L2 sees the reuse.  Inside a run, tiles go four token tiles at a time across
+    // the feature tiles: the ~64 workgroups an XCD runs concurrently then cover 4 token tiles x
+    // 16 feature tiles, which minimises what they fetch together (a token tile of activations
+    // is four times larger than a feature tile of int4 weights).
     const int total = tiles_t * tiles_n;
     int       id    = blockIdx.x;
     if (total % 8 == 0) id = (id & 7) * (total >> 3) + (id >> 3);
-    const int tile_t = id % tiles_t;
-    const int tile_n = id / tiles_t;
+    int tile_t, tile_n;
+    if (tiles_t % 4 == 0) {
+        const int r = id >> 2;
+        tile_n      = r % tiles_n;
+        tile_t      = (r / tiles_n) * 4 + (id & 3);
+    }
+    else {
+        tile_t = id % tiles_t;
+        tile_n = id / tiles_t;
+    }
     const int T0     = tile_t * TT;
     const int nt0    = (tile_n * TN) / kTileN + wave * NTW;  // first weight tile of this wave
 
