@@ -20,10 +20,11 @@ namespace w4a16 {
 namespace {
 
 constexpr int kThreads   = 256;
-#ifndef W4A16_ROWPAD
-#define W4A16_ROWPAD 16
-#endif
-constexpr int kRowHalves = kGroup + W4A16_ROWPAD;  // LDS row stride 288 bytes: measured free of bank conflicts (272 is not)
+// LDS holds two activation tiles of [tokens][128 halves] = 256 bytes per token row, i.e. 16 chunks
+// of 16 bytes.  Chunk position p of row r holds K-chunk p ^ (r & 15): the 16 lanes that read the
+// same K-chunk of 16 consecutive rows then hit 16 different bank groups, without padding, which
+// the direct global-to-LDS loads (64 lanes x 16 contiguous bytes) could not produce.
+constexpr int kRowBytes = kGroup * 2;
 
 // Compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(<N-1>); gives inline assembly
 // its immediate operands.
@@ -60,13 +61,27 @@ __device__ __forceinline__ void wait_vm(V& v)
 // Register budget: one wave per SIMD (512 registers) for the 256-register accumulator tiles,
 // two waves otherwise.  Stating it keeps the allocator from squeezing the kernel into fewer
 // VGPRs and shuttling values through AGPRs inside the loop.
+// LDS fragment read from inline assembly (byte address + immediate), and its wait.  Left to the
+// compiler, each activation fragment was read right before the two MFMAs that use it, so every
+// pair of MFMAs (32 cycles of matrix work) waited a full LDS latency.  Here a whole k32 step of
+// fragments is requested one step ahead.
+template<int OFF>
+__device__ __forceinline__ void lds_read128(half8_t& dst, uint32_t addr)
+{
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+__device__ __forceinline__ void wait_lgkm0(half8_t& v)
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v));
+}
+
 template<int TTILES, int NTW, int EPI>
 __global__ void __launch_bounds__(kThreads)
     __attribute__((amdgpu_waves_per_eu(TTILES * NTW >= 32 ? 1 : 2, TTILES * NTW >= 32 ? 1 : 2)))
 prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const uint16_t* __restrict__ X,
                const uint32_t* __restrict__ Q, const uint16_t* R_, int N, int T, int K, int tiles_t, int tiles_n)
 {
-    extern __shared__ __attribute__((aligned(16))) uint16_t xs[];  // [2][TT][kRowHalves]
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [2][TT][kRowBytes]
     constexpr int TT = 16 * TTILES;
     constexpr int TN = 64 * NTW;
 
@@ -102,15 +117,20 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     // per-thread byte offsets; the group-dependent part of every address is scalar
     const uint32_t w_off = (uint32_t)(nt0 * 1024 + lane * 16);        // + g * NT * 1024 (+ nt * 1024)
     const uint32_t q_off = (uint32_t)((nt0 * kTileN + c) * 4);        // + g * N * 4    (+ nt * 64)
-    // X staging: chunk q of this thread is row q*16 + tid/16, 16-byte column tid%16 of the tile
-    // (rows past the last token re-read the last valid row; their outputs are never stored)
-    const int xr = tid >> 4, xc = tid & 15;
-    uint32_t  x_off[TTILES];
+    // X staging, direct global -> LDS: wave w, request i writes the 1 KiB block m = w*TTILES + i
+    // (token rows 4m .. 4m+3) of the tile; lane l lands at row 4m + l/16, chunk position l%16, so it
+    // fetches K-chunk (l%16) ^ (row & 15) of that row.  Rows past the last token re-read the last
+    // valid row; their outputs are never stored.
+    uint32_t x_off[TTILES];
 #pragma unroll
-    for (int q = 0; q < TTILES; ++q)
-        x_off[q] = (uint32_t)(min(T0 + q * 16 + xr, T - 1)) * (uint32_t)(K * 2) + xc * 16;  // + g * 256
-    const int xs_w = xr * kRowHalves + xc * 8;  // + q*16*kRowHalves
-    const int xs_r = c * kRowHalves + 8 * b;    // + tt*16*kRowHalves + 32*j
+    for (int i = 0; i < TTILES; ++i) {
+        const int row = 4 * (wave * TTILES + i) + (lane >> 4);
+        x_off[i] = (uint32_t)min(T0 + row, T - 1) * (uint32_t)(K * 2) + (uint32_t)(((lane & 15) ^ (row & 15)) * 16);
+    }
+    // fragment reads: lane (c, b) reads row 16*tt + c, K-chunk 4j + b  ->  position (4j + b) ^ c
+    uint32_t xr_off[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xr_off[j] = (uint32_t)(c * kRowBytes + (((4 * j + b) ^ c) & 15) * 16);
 
     const UnpackConsts uc;
 
@@ -122,15 +142,11 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
 
     u32x4_t  wa[NTW], wb[NTW];  // weights of the current / next group (roles alternate)
     uint32_t qa[NTW], qb[NTW];
-    constexpr int XB = TTILES < 8 ? TTILES : 8;  // activation chunks staged at a time
-    u32x4_t       xst[XB];                        // activations of the next group on their way to LDS
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
         wa[nt] = wb[nt] = u32x4_t{0, 0, 0, 0};
         qa[nt] = qb[nt] = 0;
     }
-#pragma unroll
-    for (int q = 0; q < XB; ++q) xst[q] = u32x4_t{0, 0, 0, 0};
 
     auto issue_w = [&](u32x4_t (&w)[NTW], uint32_t (&qv)[NTW], int g) {
         const char* wbase = reinterpret_cast<const char*>(A) + (int64_t)g * NT * 1024;
@@ -138,41 +154,40 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         static_for<0, NTW>([&](auto nt) { gload128<nt * 1024>(w[nt], w_off, wbase); });
         static_for<0, NTW>([&](auto nt) { gload32<nt * 64>(qv[nt], q_off, qbase); });
     };
-    // activation chunks [q0, q0 + XB) of group g: request, and (later) wait for all and store
-    auto issue_x = [&](int q0, int g) {
+    // the activation tile of group g, straight into the LDS buffer `xo` (no registers, no ds_write)
+    auto issue_x = [&](uint8_t* xo, int g) {
         const char* xbase = reinterpret_cast<const char*>(X) + (int64_t)g * 256;
 #pragma unroll
-        for (int q = 0; q < XB; ++q) gload128<0>(xst[q], x_off[q0 + q], xbase);
+        for (int i = 0; i < TTILES; ++i) {
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(xbase + x_off[i]),
+                (__attribute__((address_space(3))) void*)(xo + (wave * TTILES + i) * 1024), 16, 0, 0);
+        }
     };
-    auto store_x = [&](uint16_t* xo, int q0) {
+    auto wait_all = [&](u32x4_t (&w)[NTW], uint32_t (&qv)[NTW]) {
 #pragma unroll
-        for (int q = 0; q < XB; ++q) {
-            wait_vm<0>(xst[q]);
-            *reinterpret_cast<u32x4_t*>(&xo[xs_w + (q0 + q) * 16 * kRowHalves]) = xst[q];
+        for (int nt = 0; nt < NTW; ++nt) {
+            wait_vm<0>(w[nt]);
+            wait_vm<0>(qv[nt]);
         }
     };
 
+    uint8_t* const x0 = xs;
+    uint8_t* const x1 = xs + TT * kRowBytes;
+
     // ---- prologue: group 0 ----
     issue_w(wa, qa, 0);
-#pragma unroll
-    for (int q0 = 0; q0 < TTILES; q0 += XB) {
-        issue_x(q0, 0);
-        store_x(xs, q0);
-    }
-#pragma unroll
-    for (int nt = 0; nt < NTW; ++nt) {
-        wait_vm<0>(wa[nt]);
-        wait_vm<0>(qa[nt]);
-    }
+    issue_x(x0, 0);
+    wait_all(wa, qa);
     __syncthreads();
 
     // One K step (a quantisation group): MFMAs on `w`/buffer `xb` while the next group's
     // weights go to `wn` and its activations to the other LDS buffer `xo`.
     auto step = [&](u32x4_t (&w)[NTW], uint32_t (&qv)[NTW], u32x4_t (&wn)[NTW], uint32_t (&qn)[NTW],
-                    const uint16_t* xb, uint16_t* xo, int g) {
+                    const uint8_t* xb, uint8_t* xo, int g) {
         const int gn = min(g + 1, G - 1);  // (the last step re-reads its own group: no branch)
         issue_w(wn, qn, gn);
-        issue_x(0, gn);
+        issue_x(xo, gn);
         half2_t z1024[NTW], z64[NTW], sc[NTW];
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) {
@@ -180,36 +195,36 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
             split_q(qv[nt], z1024[nt], z64[nt], s);
             sc[nt] = half2_t{s, s};
         }
+        // byte address in LDS of the tile being read
+        const uint32_t xb_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)(xb);
+        half8_t        xf[2][TTILES];  // fragments of the current / next k32 step
+        static_for<0, TTILES>([&](auto tt) { lds_read128<tt * 16 * kRowBytes>(xf[0][tt], xb_addr + xr_off[0]); });
         static_for<0, 4>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             half8_t       wf[NTW];
 #pragma unroll
             for (int nt = 0; nt < NTW; ++nt) wf[nt] = dequant_full(w[nt][j], z1024[nt], z64[nt], sc[nt], uc);
 #pragma unroll
+            for (int tt = 0; tt < TTILES; ++tt) wait_lgkm0(xf[j & 1][tt]);
+            if constexpr (j < 3) {
+                static_for<0, TTILES>([&](auto tt) {
+                    lds_read128<tt * 16 * kRowBytes>(xf[(j + 1) & 1][tt], xb_addr + xr_off[j + 1]);
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keep the requests above this step's MFMAs
+#pragma unroll
             for (int tt = 0; tt < TTILES; ++tt) {
-                const half8_t xf = *reinterpret_cast<const half8_t*>(&xb[xs_r + tt * 16 * kRowHalves + 32 * j]);
 #pragma unroll
                 for (int nt = 0; nt < NTW; ++nt)
-                    acc[tt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[nt], xf, acc[tt][nt], 0, 0, 0);
+                    acc[tt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[nt], xf[j & 1][tt], acc[tt][nt], 0, 0, 0);
             }
-            // staged activations: with 16 token tiles the first 8 chunks are stored (and the other
-            // 8 requested) after the second k32 step; the last batch is stored after the fourth
-            if constexpr (TTILES > XB && j == 1) {
-                store_x(xo, 0);
-                issue_x(XB, gn);
-            }
-            if constexpr (j == 3) store_x(xo, TTILES - XB);
         });
-#pragma unroll
-        for (int nt = 0; nt < NTW; ++nt) {  // everything has landed (vmcnt(0) above); pin the uses below it
-            wait_vm<0>(wn[nt]);
-            wait_vm<0>(qn[nt]);
-        }
+        // next group's weights are in registers and its activations in LDS once every load of this
+        // wave has completed; the barrier then publishes the other waves' parts of the tile
+        wait_all(wn, qn);
         __syncthreads();
     };
 
-    uint16_t* const x0 = xs;
-    uint16_t* const x1 = xs + TT * kRowHalves;
     int g = 0;
     for (; g + 1 < G; g += 2) {  // no branch inside: the 4*TTILES*NTW accumulators stay in place
         step(wa, qa, wb, qb, x0, x1, g);
@@ -265,7 +280,7 @@ hipError_t launch_v(const GemmArgs& a, hipStream_t st)
     constexpr int TT = 16 * TTILES, TN = 64 * NTW;
     const int     tiles_t = (a.T + TT - 1) / TT;
     const int     tiles_n = a.N / TN;
-    const size_t  lds     = (size_t)2 * TT * kRowHalves * sizeof(uint16_t);
+    const size_t  lds     = (size_t)2 * TT * kRowBytes;
     const dim3    grid(tiles_t * tiles_n), block(kThreads);
     const u32x4_t* A4 = reinterpret_cast<const u32x4_t*>(a.A);
 #define W4A16_LAUNCH(EPI)                                                                                              \
