@@ -5,6 +5,7 @@ Usage: python -m lmdeploy_amd.build            (or build_library() from Python)
 from __future__ import annotations
 
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -36,6 +37,10 @@ NO_SCRATCH = ("gemm_decode.hip", "gemm_prefill.hip")
 
 
 def _check_no_scratch(src: str, remarks: str) -> None:
+    """The GEMM kernels issue loads from inline assembly and wait for them by count, so the compiler
+    does not know when a destination register is valid.  A kernel is only safe if the compiler never
+    moves such a register: no spills to scratch, and no VGPRs parked in AGPRs (the only legitimate
+    AGPRs are the 4 * TTILES * NTW accumulators of a prefill kernel)."""
     name = None
     for line in remarks.splitlines():
         if "Function Name:" in line:
@@ -44,6 +49,13 @@ def _check_no_scratch(src: str, remarks: str) -> None:
             size = int(line.split("ScratchSize [bytes/lane]:")[1].split("[")[0])
             if size != 0:
                 raise RuntimeError("%s: kernel %s spills %d bytes/lane to scratch" % (src, name, size))
+        elif "AGPRs:" in line and name is not None and "_kernel" in name:
+            agprs = int(line.split("AGPRs:")[1].split("[")[0])
+            m = re.search(r"prefill_kernelILi(\d+)ELi(\d+)E", name)
+            allowed = 4 * int(m.group(1)) * int(m.group(2)) if m else 0
+            if agprs != allowed:
+                raise RuntimeError("%s: kernel %s uses %d AGPRs, expected %d: the register allocator is "
+                                   "parking VGPRs in AGPRs" % (src, name, agprs, allowed))
 
 
 def _compile(src: str, obj_dir: str) -> str:

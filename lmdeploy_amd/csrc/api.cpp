@@ -118,9 +118,18 @@ int algo_pick(int N, int T, int K)
 {
     if (T <= 0 || N <= 0 || K <= 0) return -1;
     if (T >= 64) {
-        // 128 x 128 tiles (two workgroups per CU hide each other's memory latency) were the
-        // fastest on every Llama shape measured; narrower token tiles for short prompts.
-        const int order[5][2] = {{128, 128}, {64, 128}, {64, 64}, {128, 256}, {256, 128}};  // tokens, features
+        // 128 x 128 tiles (two workgroups per CU) and 128 x 256 tiles (one per CU, half the LDS and
+        // L2 traffic per flop) run at about the same rate per CU; the wider tile wins when its
+        // workgroups fill the 256 CUs evenly (last round empty or more than 3/4 full), the narrower
+        // one otherwise because two small workgroups share a CU in the last round.  Narrower token
+        // tiles for short prompts.
+        bool wide = false;
+        if (N % 256 == 0 && T > 64) {
+            const int64_t wgs = (int64_t)(N / 256) * ((T + 127) / 128);
+            const int     rem = (int)(wgs % 256);
+            wide              = rem == 0 || rem > 192;
+        }
+        const int order[5][2] = {{128, wide ? 256 : 128}, {128, wide ? 128 : 256}, {64, 128}, {64, 64}, {256, 128}};  // tokens, features
         for (auto& o : order) {
             if (T <= 64 && o[0] > 64) continue;
             for (int id = 0; id < algo_count(); ++id) {

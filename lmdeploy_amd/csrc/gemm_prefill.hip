@@ -5,11 +5,19 @@
 // them straight from global memory into registers (one 128-bit load per lane and tile: the
 // tiled layout IS the MFMA operand layout), dequantises them to the reference's exact fp16
 // weight fp16_rn((q - z) * s) and uses them as the A operand of v_mfma_f32_16x16x32_f16.
-// The activations of the tile are staged once per workgroup in LDS (double buffered, one
-// 128-wide K step per quantisation group) and read as the B operand by all four waves, so
-// no weight is dequantised twice and no activation is fetched twice per workgroup.
-// With weights as A the accumulator of a lane holds four adjacent features of one token,
-// which makes every epilogue (plain, SiLU-gate on feature pairs, residual add) lane-local.
+// The activations of the tile go from global memory directly into LDS (no registers, no
+// ds_write), double buffered, one 128-wide K step per quantisation group, and are read as the
+// B operand by all four waves, so no weight is dequantised twice and no activation is fetched
+// twice per workgroup.  With weights as A the accumulator of a lane holds four adjacent
+// features of one token, which makes every epilogue (plain, SiLU-gate on feature pairs,
+// residual add) lane-local.
+//
+// The K loop is one hand-scheduled instruction stream per wave: every MFMA is followed by its
+// share of the NEXT k32 step's dequantisation, LDS fragment reads and global loads, so that a
+// single wave keeps the matrix pipe busy while it issues everything else (measured on this
+// part: an MFMA occupies the pipe for 16 cycles and issues in 4; two vector instructions fit
+// behind each one for free, a third does not).  The MFMAs are inline assembly with the
+// accumulators tied in place in AGPRs; loads are inline assembly waited for by count.
 #include "w4a16_common.h"
 #include "w4a16_internal.h"
 
@@ -58,23 +66,26 @@ __device__ __forceinline__ void wait_vm(V& v)
     asm volatile("s_waitcnt vmcnt(%1)" : "+v"(v) : "n"(N));
 }
 
-// Register budget: one wave per SIMD (512 registers) for the 256-register accumulator tiles,
-// two waves otherwise.  Stating it keeps the allocator from squeezing the kernel into fewer
-// VGPRs and shuttling values through AGPRs inside the loop.
 // LDS fragment read from inline assembly (byte address + immediate), and its wait.  Left to the
-// compiler, each activation fragment was read right before the two MFMAs that use it, so every
-// pair of MFMAs (32 cycles of matrix work) waited a full LDS latency.  Here a whole k32 step of
-// fragments is requested one step ahead.
+// compiler, each activation fragment was read right before the MFMAs that use it, which then
+// waited a full LDS latency; and any compiler-visible LDS read after a direct-to-LDS load would
+// be preceded by a wait for ALL loads in flight.  Here the fragments of a k32 step are requested
+// during the previous one.
 template<int OFF>
 __device__ __forceinline__ void lds_read128(half8_t& dst, uint32_t addr)
 {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
-__device__ __forceinline__ void wait_lgkm0(half8_t& v)
+__device__ __forceinline__ void wait_lgkm0(half8_t& a, half8_t& b, half8_t& c, half8_t& d)
 {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v));
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
 }
 
+// Register budget: one wave per SIMD (512 registers) for the 128-register accumulator tiles,
+// two waves otherwise.  Stating it keeps the allocator from squeezing the kernel into fewer
+// VGPRs and parking values in AGPRs, which is fatal here: a register parked while an
+// inline-assembly load into it is still in flight is handed to another value, and the load then
+// lands on that value (the build rejects kernels that use AGPRs beyond their accumulators).
 template<int TTILES, int NTW, int EPI>
 __global__ void __launch_bounds__(kThreads)
     __attribute__((amdgpu_waves_per_eu(TTILES * NTW >= 32 ? 1 : 2, TTILES * NTW >= 32 ? 1 : 2)))
@@ -164,6 +175,24 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
                 (__attribute__((address_space(3))) void*)(xo + (wave * TTILES + i) * 1024), 16, 0, 0);
         }
     };
+    // the same requests one at a time (m = 0 .. 2 NTW + TTILES - 1), to be dealt out between MFMAs
+    constexpr int kVmOps = 2 * NTW + TTILES;
+    auto vm_op = [&](auto M, u32x4_t (&w)[NTW], uint32_t (&qv)[NTW], uint8_t* xo, const char* wbase, const char* qbase,
+                     const char* xbase) {
+        constexpr int m = decltype(M)::value;
+        if constexpr (m < NTW) {
+            gload128<m * 1024>(w[m], w_off, wbase);
+        }
+        else if constexpr (m < 2 * NTW) {
+            gload32<(m - NTW) * 64>(qv[m - NTW], q_off, qbase);
+        }
+        else {
+            constexpr int i = m - 2 * NTW;
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(xbase + x_off[i]),
+                (__attribute__((address_space(3))) void*)(xo + (wave * TTILES + i) * 1024), 16, 0, 0);
+        }
+    };
     auto wait_all = [&](u32x4_t (&w)[NTW], uint32_t (&qv)[NTW]) {
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) {
@@ -175,62 +204,139 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     uint8_t* const x0 = xs;
     uint8_t* const x1 = xs + TT * kRowBytes;
 
-    // ---- prologue: group 0 ----
-    issue_w(wa, qa, 0);
-    issue_x(x0, 0);
-    wait_all(wa, qa);
-    __syncthreads();
+    // State carried from one k32 step to the next (and across K steps): dequantised weights and
+    // activation fragments of the current / next k32 step, zero points and scale of the current /
+    // next group.
+    half8_t wf[2][NTW];
+    half8_t xf[2][TTILES];
+    half2_t z1024[2][NTW], z64[2][NTW], sc[2][NTW];
 
-    // One K step (a quantisation group): MFMAs on `w`/buffer `xb` while the next group's
-    // weights go to `wn` and its activations to the other LDS buffer `xo`.
-    auto step = [&](u32x4_t (&w)[NTW], uint32_t (&qv)[NTW], u32x4_t (&wn)[NTW], uint32_t (&qn)[NTW],
-                    const uint8_t* xb, uint8_t* xo, int g) {
-        const int gn = min(g + 1, G - 1);  // (the last step re-reads its own group: no branch)
-        issue_w(wn, qn, gn);
-        issue_x(xo, gn);
-        half2_t z1024[NTW], z64[NTW], sc[NTW];
+    auto split = [&](auto P_, uint32_t (&qv)[NTW]) {
+        constexpr int P = decltype(P_)::value;
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) {
             half_t s;
-            split_q(qv[nt], z1024[nt], z64[nt], s);
-            sc[nt] = half2_t{s, s};
+            split_q(qv[nt], z1024[P][nt], z64[P][nt], s);
+            sc[P][nt] = half2_t{s, s};
         }
-        // byte address in LDS of the tile being read
-        const uint32_t xb_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)(xb);
-        half8_t        xf[2][TTILES];  // fragments of the current / next k32 step
-        static_for<0, TTILES>([&](auto tt) { lds_read128<tt * 16 * kRowBytes>(xf[0][tt], xb_addr + xr_off[0]); });
+    };
+    // The dequantisation of word J of every tile of `w`, as 13 * NTW single vector instructions
+    // (op = NTW * k + nt) so that they can be dealt out between the MFMAs of a k32 step:
+    // k = 0: w >> 8;  1..4: (w & mask) | magic;  5..8: - (offset + zero);  9..12: * scale.
+    uint32_t dq[NTW][5];
+    auto dequant_op = [&](auto P, auto J, auto OP, u32x4_t (&w)[NTW]) {
+        constexpr int p = decltype(P)::value, j = decltype(J)::value;
+        constexpr int nt = decltype(OP)::value % NTW, k = decltype(OP)::value / NTW;
+        if constexpr (k == 0) dq[nt][4] = w[nt][j] >> 8;
+        else if constexpr (k <= 4) {
+            constexpr int i  = k - 1;
+            const uint32_t src = i < 2 ? w[nt][j] : dq[nt][4];
+            dq[nt][i] = (src & (i & 1 ? uc.mask_hi : uc.mask_lo)) | (i & 1 ? uc.magic_hi : uc.magic_lo);
+        }
+        else if constexpr (k <= 8) {
+            constexpr int i = k - 5;
+            dq[nt][i]       = as_u32(as_half2(dq[nt][i]) - (i & 1 ? z64[p][nt] : z1024[p][nt]));
+        }
+        else {
+            constexpr int i = k - 9;
+            const half2_t r = as_half2(dq[nt][i]) * sc[p][nt];
+            wf[j & 1][nt][2 * i]     = r[0];
+            wf[j & 1][nt][2 * i + 1] = r[1];
+        }
+    };
+    auto dequant = [&](auto P, auto J, u32x4_t (&w)[NTW]) {
+        static_for<0, 13 * NTW>([&](auto op) { dequant_op(P, J, op, w); });
+    };
+    auto read_x = [&](auto J_, const uint8_t* xb) {
+        constexpr int  J    = decltype(J_)::value;
+        const uint32_t addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)(xb) + xr_off[J];
+        static_for<0, TTILES>([&](auto tt) { lds_read128<tt * 16 * kRowBytes>(xf[J & 1][tt], addr); });
+    };
+    auto read_x1 = [&](auto J_, auto TT_, uint32_t base) {
+        constexpr int J = decltype(J_)::value, tt = decltype(TT_)::value;
+        lds_read128<tt * 16 * kRowBytes>(xf[J & 1][tt], base + xr_off[J]);
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+
+    // ---- prologue: groups 0 and 1 in flight, first operands of group 0 prepared ----
+    issue_w(wa, qa, 0);
+    issue_x(x0, 0);
+    issue_w(wb, qb, min(1, G - 1));
+    issue_x(x1, min(1, G - 1));
+    wait_all(wa, qa);
+    wait_all(wb, qb);
+    __syncthreads();
+    read_x(I0{}, x0);
+    split(I0{}, qa);
+    dequant(I0{}, I0{}, wa);
+
+    // One K step (a quantisation group, four k32 steps) on the weights `w` (group parity P) and the
+    // LDS buffer `xb`.  Every k32 step runs its MFMAs interleaved with the dequantisation of the
+    // NEXT k32 step's weights and the requests for its activation fragments.  In the last k32 step
+    // the next group's weights (`wn`, requested one K step ago) and activation tile (`xo`) are
+    // complete: the workgroup synchronises, starts on them, and re-uses `w` and `xb`, which no wave
+    // reads any more, for the loads of group g + 2.
+    auto step = [&](auto P, u32x4_t (&w)[NTW], uint32_t (&qv)[NTW], u32x4_t (&wn)[NTW], uint32_t (&qn)[NTW],
+                    uint8_t* xb, const uint8_t* xo, int g) {
+        constexpr int p  = decltype(P)::value;
+        using PN         = std::integral_constant<int, p ^ 1>;
         static_for<0, 4>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            half8_t       wf[NTW];
+            using JN        = std::integral_constant<int, (j + 1) & 3>;
 #pragma unroll
-            for (int nt = 0; nt < NTW; ++nt) wf[nt] = dequant_full(w[nt][j], z1024[nt], z64[nt], sc[nt], uc);
-#pragma unroll
-            for (int tt = 0; tt < TTILES; ++tt) wait_lgkm0(xf[j & 1][tt]);
-            if constexpr (j < 3) {
-                static_for<0, TTILES>([&](auto tt) {
-                    lds_read128<tt * 16 * kRowBytes>(xf[(j + 1) & 1][tt], xb_addr + xr_off[j + 1]);
+            for (int tt = 0; tt < TTILES; tt += 4)
+                wait_lgkm0(xf[j & 1][tt], xf[j & 1][tt + 1], xf[j & 1][tt + 2], xf[j & 1][tt + 3]);
+            const int   g2 = min(g + 2, G - 1);  // (the last steps re-read the last group: no branch)
+            const char* wbase = reinterpret_cast<const char*>(A) + (int64_t)g2 * NT * 1024;
+            const char* qbase = reinterpret_cast<const char*>(Q) + (int64_t)g2 * N * 4;
+            const char* xbase = reinterpret_cast<const char*>(X) + (int64_t)g2 * 256;
+            if constexpr (j == 3) {
+                wait_all(wn, qn);
+                __syncthreads();
+            }
+            const uint32_t rbase =
+                (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)(j < 3 ? (const uint8_t*)xb : xo);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (j == 3) split(PN{}, qn);
+            // one MFMA, then its share of the next k32 step's dequantisation, and so on
+            constexpr int kOps = 13 * NTW, kSlots = TTILES * NTW;
+            static_for<0, kSlots>([&](auto ic) {
+                constexpr int i = decltype(ic)::value, tt = i / NTW, nt = i % NTW;
+                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
+                             : "+a"(acc[tt][nt])
+                             : "v"(wf[j & 1][nt]), "v"(xf[j & 1][tt]));
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<i * kOps / kSlots, (i + 1) * kOps / kSlots>([&](auto op) {
+                    if constexpr (j < 3) dequant_op(P, JN{}, op, w);
+                    else dequant_op(PN{}, I0{}, op, wn);
                 });
-            }
-            __builtin_amdgcn_sched_barrier(0);  // keep the requests above this step's MFMAs
-#pragma unroll
-            for (int tt = 0; tt < TTILES; ++tt) {
-#pragma unroll
-                for (int nt = 0; nt < NTW; ++nt)
-                    acc[tt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[nt], xf[j & 1][tt], acc[tt][nt], 0, 0, 0);
-            }
+                // the next k32 step's activation fragments, requested during the first three quarters
+                // of this one; in the last k32 step also the loads of group g + 2
+                constexpr int kR = kSlots * 3 / 4 > 0 ? kSlots * 3 / 4 : 1;
+                if constexpr (i < kR) {
+                    static_for<i * TTILES / kR, (i + 1) * TTILES / kR>([&](auto tt) { read_x1(JN{}, tt, rbase); });
+                }
+                if constexpr (j == 3) {
+                    static_for<i * kVmOps / kSlots, (i + 1) * kVmOps / kSlots>(
+                        [&](auto m) { vm_op(m, w, qv, xb, wbase, qbase, xbase); });
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
         });
-        // next group's weights are in registers and its activations in LDS once every load of this
-        // wave has completed; the barrier then publishes the other waves' parts of the tile
-        wait_all(wn, qn);
-        __syncthreads();
     };
 
     int g = 0;
     for (; g + 1 < G; g += 2) {  // no branch inside: the 4*TTILES*NTW accumulators stay in place
-        step(wa, qa, wb, qb, x0, x1, g);
-        step(wb, qb, wa, qa, x1, x0, g + 1);
+        step(I0{}, wa, qa, wb, qb, x0, x1, g);
+        step(I1{}, wb, qb, wa, qa, x1, x0, g + 1);
     }
-    if (g < G) step(wa, qa, wb, qb, x0, x1, g);
+    if (g < G) step(I0{}, wa, qa, wb, qb, x0, x1, g);
+    wait_all(wa, qa);  // no load may still be writing LDS or registers when the wave ends
+    wait_all(wb, qb);
+    // the MFMAs are inline assembly, so the compiler does not know that the accumulators are
+    // still being written: cover the longest MFMA-result-to-VALU-read distance by hand
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
     // ---- epilogue: lane (c, b) of tile (tt, nt) holds token T0 + 16 tt + c, features n .. n+3 ----
 #pragma unroll
