@@ -43,7 +43,7 @@ typedef struct w4a16_metric {
     int   id;          /* algo_id accepted by w4a16_gemm                        */
     int   feasible;    /* 1 if the kernel can run this shape                    */
     int   best;        /* 1 for the algo the heuristic (algo_id < 0) would pick */
-    int   kind;        /* 0 = decode (skinny) kernel, 1 = MFMA prefill kernel   */
+    int   kind;        /* 0 = decode kernel (column blocks), 1 = MFMA prefill kernel, 2 = decode kernel (strips) */
     int   tile_n;      /* output features per workgroup                         */
     int   tile_t;      /* tokens per workgroup                                  */
     int   slices;      /* decode: K slices (wave groups) per workgroup            */

@@ -6,6 +6,12 @@ import ctypes
 import os
 from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_size_t, c_void_p
 
+# The callers hand over torch tensors, so torch is in the process anyway - and it must come first:
+# torch ships its own libamdhip64 and libw4a16.so has to bind to that same HIP runtime.  Loaded the
+# other way round, the system runtime gets in first, two runtimes share the process, and the first
+# kernel launch reports "no ROCm-capable device is detected".
+import torch  # noqa: F401  (imported for its side effect on the dynamic loader)
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # W4A16_LIB overrides the in-tree library (e.g. to try a differently tuned build)
 LIB_PATH = os.environ.get("W4A16_LIB") or os.path.join(_HERE, "lib", "libw4a16.so")

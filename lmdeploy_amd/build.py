@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libw4a16.so")
 
-SOURCES = ["api.cpp", "repack.hip", "gemm_decode.hip", "gemm_prefill.hip"]
+SOURCES = ["api.cpp", "repack.hip", "gemm_decode.hip", "gemm_strip.hip", "gemm_prefill.hip"]
 
 # -packed-fp32-ops off: hipcc must not form v_pk_*_f32 instructions for this target.
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
@@ -33,7 +33,7 @@ def _hipcc() -> str:
 # The GEMM kernels wait for their software-pipelined loads by count.  A register spill would put
 # scratch stores among those loads, and stores complete out of order with loads, so a spilling
 # GEMM kernel is a wrong kernel: the build refuses it.
-NO_SCRATCH = ("gemm_decode.hip", "gemm_prefill.hip")
+NO_SCRATCH = ("gemm_decode.hip", "gemm_strip.hip", "gemm_prefill.hip")
 
 
 def _check_no_scratch(src: str, remarks: str) -> None:
@@ -58,6 +58,26 @@ def _check_no_scratch(src: str, remarks: str) -> None:
                                    "parking VGPRs in AGPRs" % (src, name, agprs, allowed))
 
 
+def _check_inflight(src: str, obj_dir: str) -> None:
+    """Second pass over the same source to assembly text, checked by asm_lint: no compiler-generated
+    instruction may touch a register whose inline-assembly load can still be in flight."""
+    try:
+        from .asm_lint import lint
+    except ImportError:  # run as a script
+        from asm_lint import lint
+    asm = os.path.join(obj_dir, os.path.splitext(src)[0] + ".s")
+    cmd = [_hipcc(), *HIP_FLAGS, "-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", asm]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc -S failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
+    with open(asm) as f:
+        problems = lint(f.read())
+    os.remove(asm)
+    if problems:
+        raise RuntimeError("%s: %d uses of registers with a load in flight, e.g.\n%s"
+                           % (src, len(problems), "\n".join(problems[:5])))
+
+
 def _compile(src: str, obj_dir: str) -> str:
     obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
     cmd = [_hipcc(), *HIP_FLAGS]
@@ -71,6 +91,7 @@ def _compile(src: str, obj_dir: str) -> str:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
     if src in NO_SCRATCH:
         _check_no_scratch(src, r.stderr)
+        _check_inflight(src, obj_dir)
     return obj
 
 
@@ -79,7 +100,7 @@ def build_library(verbose: bool = True) -> str:
     obj_dir = os.path.join(HERE, "build")
     os.makedirs(obj_dir, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(5, len(SOURCES))) as ex:
         objs = list(ex.map(lambda s: _compile(s, obj_dir), SOURCES))
     tmp = LIB_PATH + ".tmp"
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]

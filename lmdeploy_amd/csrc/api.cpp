@@ -66,6 +66,8 @@ std::vector<Algo> build_table()
         t.push_back(Algo{0, 64, 16, 1, 0, DecodeConfig{1, 4, 1, 4, fill}});
         t.push_back(Algo{0, 128, 16, 2, 0, DecodeConfig{1, 8, 2, 4, fill}});
     }
+    // strips of column tiles over the whole of K, 1 or 2 per CU
+    for (int per_cu : {1, 2}) t.push_back(Algo{2, 0, 16, 8, per_cu, DecodeConfig{}});
     for (int v = 0; v < prefill_variants(); ++v) {
         int tn = 0, tt = 0;
         prefill_tile(v, tn, tt);
@@ -95,18 +97,21 @@ const Algo& algo_at(int id)
 bool algo_feasible(int id, int N, int T, int K)
 {
     const Algo& a = algo_at(id);
+    if (a.kind == 2) return strip_feasible(a.param, N, T, K);
     return a.kind == 0 ? decode_feasible(a.dc, N, T, K) : prefill_feasible(a.param, N, T, K);
 }
 
 int algo_grid(int id, int N, int T, int K, const Scratch& sc)
 {
     const Algo& a = algo_at(id);
+    if (a.kind == 2) return strip_grid(a.param, N, T, K);
     return a.kind == 0 ? decode_grid(a.dc, N, T, K, sc.ws_bytes, sc.cnt_len) : prefill_grid(a.param, N, T, K);
 }
 
 hipError_t algo_launch(int id, const GemmArgs& g, const Scratch& sc, hipStream_t st)
 {
     const Algo& a = algo_at(id);
+    if (a.kind == 2) return strip_launch(a.param, g, st);
     return a.kind == 0 ? decode_launch(a.dc, g, sc.ws, sc.ws_bytes, sc.cnt, sc.cnt_len, st) :
                          prefill_launch(a.param, g, st);
 }
@@ -140,10 +145,21 @@ int algo_pick(int N, int T, int K)
         for (int id = 0; id < algo_count(); ++id)
             if (algo_at(id).kind == 1 && algo_feasible(id, N, T, K)) return id;
     }
-    // Decode: one column tile per wave, four groups in flight.  Wide matrices give every wave its
-    // own column tiles and share the activations among eight waves; narrow ones also slice K
-    // inside the workgroup so that at least 256 workgroups exist.  (From sweeps on MI355X.)
-    const int nt = N / 16, groups = K / 128;
+    // Decode.  Strips of column tiles over the whole of K, one per CU, were the fastest on every
+    // Llama-7B/70B shape measured at 1..16 tokens; two narrower strips per CU are slightly ahead on
+    // very wide matrices while the activations are small.  Matrices with too few column tiles to
+    // give every CU a strip fall back to the column-block kernel, which can also split K across
+    // workgroups.
+    if (N / 16 >= 128) {
+        const int want = (N / 16 >= 1024 && T <= 8) ? 2 : 1;
+        for (int per_cu : {want, 1}) {
+            for (int id = 0; id < algo_count(); ++id) {
+                const Algo& a = algo_at(id);
+                if (a.kind == 2 && a.param == per_cu && algo_feasible(id, N, T, K)) return id;
+            }
+        }
+    }
+    // Column-block kernel: one column tile per wave, four groups in flight.    const int nt = N / 16, groups = K / 128;
     int       wn, sk, fill = 0;
     if (nt >= 1024) {
         wn = 8, sk = 1;
@@ -190,6 +206,7 @@ int check_gemm_args(const w4a16_handle* h, const void* C, const void* A, const v
         (reinterpret_cast<uintptr_t>(Q) & 3u) || (R && (reinterpret_cast<uintptr_t>(R) & 3u)))
         return fail(W4A16_EARG, "misaligned pointer (A and X need 16 bytes, C, Q, R need 4)");
     if (k == 0 || k % 128 != 0 || n_out % 16 != 0) return fail(W4A16_ESHAPE, "no feasible kernel found");
+    (void)hipGetLastError();  // an error some earlier caller left behind is not this launch's
     return 0;
 }
 
@@ -272,7 +289,7 @@ int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const 
         w4a16_metric m{};
         m.id       = id;
         m.kind     = a.kind;
-        m.tile_n   = a.tile_n;
+        m.tile_n   = a.kind == 2 ? 16 * strip_width(a.param, n_out, tokens, k) : a.tile_n;
         m.tile_t   = a.tile_t;
         m.slices   = a.slices;
         m.best     = id == best;
@@ -308,6 +325,7 @@ static int check_repack(const char* what, int m, int k, int m_mult, int k_mult)
     if (m < 0 || k < 0) return fail(W4A16_EARG, "%s: negative size", what);
     if (m % m_mult != 0 || k % k_mult != 0)
         return fail(W4A16_ESHAPE, "%s: m must be a multiple of %d and k of %d (got m=%d k=%d)", what, m_mult, k_mult, m, k);
+    (void)hipGetLastError();  // an error some earlier caller left behind is not this launch's
     return 0;
 }
 

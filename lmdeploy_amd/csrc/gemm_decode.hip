@@ -10,11 +10,15 @@
 // almost only weight bytes.  Slice partial sums are added in LDS in slice order.
 //
 // Per group and column tile a wave computes accg[t, n] = sum_k X[t, k] * (q[k, n] - z[n])
-// with four v_mfma_f32_16x16x32_f16 (activations = A operand, de-offset int4 = B operand;
-// the differences are exact in fp16), then acc += s[n] * accg in fp32.  Scaling after the
-// group sum keeps the per-weight multiply out of the inner loop (9 VALU instructions per 8
-// weights).  The result differs from "round every weight to fp16 first" only by that rounding
-// (<= 2^-11 relative per term).
+// with v_mfma_f32_16x16x32_f16 (activations = A operand), then acc += s[n] * accg in fp32.
+// The B operand of four MFMAs is the unpacked int4 still carrying its fp16 offset (1024 + q
+// or 64 + q: 5 VALU instructions per 8 weights); four more MFMAs on a B operand that is
+// -(offset + z) everywhere take the offsets and the zero point out again.  Every product is
+// exact in fp32 and the matrix pipe is idle most of the time anyway, whereas the vector ALU is
+// what bounds this kernel on large matrices.  Scaling after the group sum keeps the per-weight
+// multiply out of the inner loop.  The result differs from "round every weight to fp16
+// first" by that rounding (<= 2^-11 relative per term) and by the fp32 rounding of sums that
+// carry the offsets (<= 2^-24 * 1039 * sum|x| per group, before scaling).
 //
 // Split K across workgroups (SK > 1, used only when a matrix has too few column tiles to
 // fill the chip otherwise): every workgroup writes its fp32 partial tiles to a workspace,
@@ -166,19 +170,32 @@ decode_kernel(const DecodeParams p)
         for (int j = 0; j < 4; ++j) xf[j] = __builtin_bit_cast(half8_t, xs_me[gl * kSlots + j * 4 * TP]);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            half2_t z1024, z64;
-            half_t  sc;
-            split_q(s.q[r], z1024, z64, sc);
+            // B operand that removes the unpack offsets and the zero point: -(1024 + z) under the
+            // low-nibble pairs, -(64 + z) under the high-nibble pairs.  One MFMA with it per k32
+            // step replaces four packed subtractions per weight word on the vector ALU, which is
+            // the unit this kernel saturates; all products are exact and the sums are fp32.
+            const half2_t h   = as_half2(s.q[r]);
+            const half2_t n64 = half2_t{h[0], h[0]} * half2_t{(half_t)-1.f, (half_t)-1.f};
+            const uint32_t zb = ((s.q[r] >> 4) & 0xfu) * 0x10001u + 0xE400E400u;  // -(1024 + z) twice
+            half8_t bz;
+            bz[0] = as_half2(zb)[0]; bz[1] = as_half2(zb)[1]; bz[2] = n64[0]; bz[3] = n64[1];
+            bz[4] = bz[0]; bz[5] = bz[1]; bz[6] = bz[2]; bz[7] = bz[3];
             // Convert the scale now and hide it from the optimiser: otherwise the conversion is
             // folded into the final multiply-add, the Q word stays live past the refill of this
             // stage, and the refill needs a copy that waits for every load in flight.
-            float sf = (float)sc;
+            float sf = (float)h[1];
             asm volatile("" : "+v"(sf));
             float4_t g4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
+            for (int j = 0; j < 4; ++j) g4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[j], bz, g4, 0, 0, 0);
+#pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const half8_t wf = dequant_sub(s.w[r][j], z1024, z64, uc);
-                g4               = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[j], wf, g4, 0, 0, 0);
+                uint32_t v[4];
+                unpack_offset(s.w[r][j], v, uc);
+                half8_t wf;
+                wf[0] = as_half2(v[0])[0]; wf[1] = as_half2(v[0])[1]; wf[2] = as_half2(v[1])[0]; wf[3] = as_half2(v[1])[1];
+                wf[4] = as_half2(v[2])[0]; wf[5] = as_half2(v[2])[1]; wf[6] = as_half2(v[3])[0]; wf[7] = as_half2(v[3])[1];
+                g4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[j], wf, g4, 0, 0, 0);
             }
             acc[r] += sf * g4;
         }

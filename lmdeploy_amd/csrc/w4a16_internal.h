@@ -27,11 +27,11 @@ struct DecodeConfig {
 };
 
 struct Algo {
-    int          kind;     // 0 decode, 1 prefill
+    int          kind;     // 0 decode (column blocks), 1 prefill, 2 decode (strips)
     int          tile_n;   // output features per workgroup
     int          tile_t;   // tokens per workgroup
     int          slices;   // K slices per workgroup
-    int          param;    // prefill: variant index
+    int          param;    // prefill: variant index; strips: strips per CU aimed for
     DecodeConfig dc;       // decode only
 };
 
@@ -69,6 +69,12 @@ bool       decode_feasible(const DecodeConfig& cf, int N, int T, int K);
 int        decode_grid(const DecodeConfig& cf, int N, int T, int K, size_t ws_bytes, int cnt_len);
 hipError_t decode_launch(const DecodeConfig& cf, const GemmArgs& a, float* ws, size_t ws_bytes, int* cnt, int cnt_len,
                          hipStream_t st);
+
+// decode kernels, strip decomposition (gemm_strip.hip)
+bool       strip_feasible(int per_cu, int N, int T, int K);
+int        strip_grid(int per_cu, int N, int T, int K);
+int        strip_width(int per_cu, int N, int T, int K);  // column tiles of the widest strip
+hipError_t strip_launch(int per_cu, const GemmArgs& a, hipStream_t st);
 
 // MFMA prefill kernels
 int        prefill_variants();

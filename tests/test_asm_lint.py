@@ -1,0 +1,48 @@
+"""The build-time assembly check must catch a register that is touched while an inline-assembly
+load into it is still in flight, and must accept the same code once a counted wait covers it."""
+from lmdeploy_amd.asm_lint import lint
+
+HEAD = "_ZN5w4a164test_kernelEv:\n"
+TAIL = "\ts_endpgm\n.Lfunc_end0:\n"
+
+
+def load(reg):
+    return "\t;;#ASMSTART\n\tglobal_load_dwordx4 v[%d:%d], v40, s[2:3] offset:0\n\t;;#ASMEND\n" % (reg, reg + 3)
+
+
+def test_clean_counted_wait():
+    asm = HEAD + load(0) + load(4) + "\ts_waitcnt vmcnt(1)\n\tv_mov_b32_e32 v20, v1\n" + TAIL
+    assert lint(asm) == []
+
+
+def test_copy_before_wait_is_reported():
+    asm = HEAD + load(0) + load(4) + "\tv_mov_b32_e32 v20, v1\n\ts_waitcnt vmcnt(1)\n" + TAIL
+    msgs = lint(asm)
+    assert len(msgs) == 1 and "v1" in msgs[0]
+
+
+def test_wait_too_weak_is_reported():
+    # vmcnt(1) retires only the older load: v[4:7] may still be in flight
+    asm = HEAD + load(0) + load(4) + "\ts_waitcnt vmcnt(1)\n\tv_add_u32_e32 v21, v5, v5\n" + TAIL
+    assert len(lint(asm)) == 1
+
+
+def test_loop_carried_load_is_tracked_across_the_back_edge():
+    # the load at the end of the loop body is in flight at the top of the next trip
+    asm = (HEAD + load(0) + ".LBB0_1:\n\ts_waitcnt vmcnt(0)\n\tv_mov_b32_e32 v20, v0\n" + load(0)
+           + "\tv_mov_b32_e32 v21, v2\n\ts_cbranch_scc1 .LBB0_1\n" + TAIL)
+    msgs = lint(asm)
+    assert len(msgs) == 1 and "v_mov_b32_e32 v21, v2" in msgs[0]
+
+
+def test_join_takes_the_younger_position():
+    # one path issues a second load, so after the join vmcnt(1) no longer covers v[0:3]... it does:
+    # v[0:3] is older on both paths; v[4:7] is only in flight on one of them and must stay flagged
+    asm = (HEAD + load(0) + "\ts_cbranch_scc1 .LBB0_2\n" + load(4) + ".LBB0_2:\n\ts_waitcnt vmcnt(1)\n"
+           "\tv_mov_b32_e32 v20, v4\n" + TAIL)
+    assert len(lint(asm)) == 1
+
+
+def test_other_functions_are_ignored():
+    asm = "_ZN5w4a166helperEv:\n" + load(0) + "\tv_mov_b32_e32 v20, v1\n" + TAIL
+    assert lint(asm) == []
