@@ -159,7 +159,10 @@ int algo_pick(int N, int T, int K)
             }
         }
     }
-    // Column-block kernel: one column tile per wave, four groups in flight.    const int nt = N / 16, groups = K / 128;
+    // Column-block kernel: one column tile per wave, four groups in flight.  Wide matrices give
+    // every wave its own column tiles and share the activations among eight waves; narrow ones
+    // also slice K inside the workgroup so that at least 256 workgroups exist.
+    const int nt = N / 16, groups = K / 128;
     int       wn, sk, fill = 0;
     if (nt >= 1024) {
         wn = 8, sk = 1;
