@@ -31,8 +31,8 @@ MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16 matrix
 # HBM bytes per launch of the two dominant kernels, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
 # runs of `bench.py --probe ...`, calibrated against an elementwise kernel of known size
 # (profiles/decode_gate_up_hbm_traffic.md, profiles/prefill_gate_up_mfma_and_traffic.md).
-TRAFFIC_DECODE_GATE_UP = 48.66e6
-TRAFFIC_PREFILL_GATE_UP = 558.7e6
+TRAFFIC_DECODE_GATE_UP = 49.36e6
+TRAFFIC_PREFILL_GATE_UP = 564.4e6
 
 # name, K, N (gate_up: both halves), epilogue
 LAYER_7B = [("qkv", 4096, 12288, 0), ("o", 4096, 4096, 0), ("gate_up", 4096, 22016, 1), ("down", 11008, 4096, 2)]
@@ -184,7 +184,7 @@ def main():
     achieved = gu_bytes / (gu_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_DECODE_GATE_UP,
-                "kernel": "decode_kernel, gate_up K=4096 N=22016 +SiLU, T cycling over {1,4,8,16}",
+                "kernel": "strip_kernel, gate_up K=4096 N=22016 +SiLU, T cycling over {1,4,8,16}",
                 "bytes_per_launch": int(gu_bytes), "us_per_launch": round(gu_us, 3)}
 
     # ---- per-shape decode table ----------------------------------------------------------------
