@@ -247,6 +247,89 @@ def test_llama7b_prefill_shapes_sampled_rows(tm, gemm, name, K, N, kind):
     assert np.isfinite(got).all() and err <= TOL, (name, err)
 
 
+LLAMA70B = [("qkv70", 8192, 10240, 0), ("o70", 8192, 8192, 0), ("gate_up70", 8192, 57344, 1), ("down70", 28672, 8192, 2)]
+
+
+@pytest.mark.parametrize("name,K,N,kind", LLAMA70B)
+def test_llama70b_shapes_sampled_columns(tm, gemm, name, K, N, kind):
+    """Llama-2-70B GQA layer shapes, unsharded, at M in {1, 16, 2048}.  The GPU computes everything;
+    the oracle dequantises 512 sampled column pairs (first, last and random ones: output columns are
+    independent, and pairs keep gate/up together for the SiLU epilogue) and, at 2048 tokens, 48
+    sampled token rows."""
+    Tmax = 2048
+    d = O.make_inputs(700 + kind + K // 1024, Tmax, K, N, residual=kind == 2)
+    A, Q = convert(tm, d, N, K)
+    rng = np.random.default_rng(5)
+    pairs = np.unique(np.concatenate([[0, 1, 7, 8, N // 2 - 1], rng.integers(0, N // 2, 507)]))
+    cols = np.stack([2 * pairs, 2 * pairs + 1], axis=1).reshape(-1)
+    Wc = O.dequant_weights(d["q"][:, cols], d["z"][:, cols], d["scales"][:, cols], 128)
+    for T in (1, 16, Tmax):
+        dd = dict(d, X=d["X"][:T])
+        if kind == 2:
+            dd["R"] = d["R"][:T]
+        got = run(tm, gemm, dd, A, Q, T, K, N, kind)
+        rows = np.arange(T) if T <= 16 else np.unique(np.concatenate([[0, 15, 16, T - 1], rng.integers(0, T, 44)]))
+        want = O.epilogue(O.gemm_acc(dd["X"][rows], Wc), kind, dd["R"][rows][:, cols] if kind == 2 else None)
+        sel = got[rows][:, pairs] if kind == 1 else got[rows][:, cols]
+        err = O.max_abs_rel(sel, want)
+        assert np.isfinite(got).all() and err <= TOL, (name, T, err)
+
+
+def test_llama7b_32_layer_decode_sequence(tm, gemm):
+    """The full 32-layer Llama-2-7B GEMM sequence of one decode step at M = 8: per layer
+    qkv -> o -> gate_up (SiLU) -> down (+ residual), every layer with its own random int4 weights
+    (3.5 GB packed), outputs feeding the next GEMM.  Attention and norms are not part of this path:
+    o_proj reads the first 4096 features of the qkv output, and every GEMM input is rescaled to unit
+    variance on the host side of the test so that 128 chained GEMMs stay in fp16 range.  The oracle
+    replays layers 0 and 31 from the GPU's own inputs to those layers."""
+    T, H, F, L = 8, 4096, 11008, 32
+    gen = torch.Generator(device="cuda").manual_seed(1234)
+
+    def rand_w(K, N):
+        A = torch.randint(-2 ** 31, 2 ** 31 - 1, (K * N // 8,), dtype=torch.int32, device="cuda", generator=gen)
+        s = (torch.randn((K // 128, N), device="cuda", generator=gen).abs() * 0.01 + 1e-3).half()
+        z = torch.randint(0, 16, (K // 128, N), device="cuda", generator=gen, dtype=torch.int32)
+        Q = (s.view(torch.int16).to(torch.int32) << 16) | (0x5400 | (z << 4))
+        return A, Q
+
+    shapes = [(H, 3 * H, 0), (H, H, 0), (H, 2 * F, 1), (F, H, 2)]
+    layers = [[rand_w(K, N) for K, N, _ in shapes] for _ in range(L)]
+    x = torch.randn(T, H, device="cuda", generator=gen).half()
+    keep = {}
+
+    def norm(t):
+        return (t.float() / t.float().std()).half()
+
+    for li, ws in enumerate(layers):
+        x_in = norm(x)
+        qkv = torch.empty(T, 3 * H, dtype=torch.float16, device="cuda")
+        gemm.Run(qkv, ws[0][0], x_in, ws[0][1], 3 * H, T, H, 128, 0)
+        o_in = norm(qkv[:, :H]).contiguous()
+        o = torch.empty(T, H, dtype=torch.float16, device="cuda")
+        gemm.Run(o, ws[1][0], o_in, ws[1][1], H, T, H, 128, 0)
+        f_in = norm(o)
+        act = torch.empty(T, F, dtype=torch.float16, device="cuda")
+        gemm.Run(act, ws[2][0], f_in, ws[2][1], 2 * F, T, H, 128, 1)
+        d_in = norm(act)
+        out = x_in.clone()
+        gemm.Run(out, ws[3][0], d_in, ws[3][1], H, T, F, 128, 2, -1, residual=out)
+        if li in (0, L - 1):
+            keep[li] = [t.cpu().numpy() for t in (x_in, qkv, o_in, o, f_in, act, d_in, out)]
+        x = out
+    torch.cuda.synchronize()
+    assert torch.isfinite(x).all()
+
+    for li in (0, L - 1):
+        x_in, qkv, o_in, o, f_in, act, d_in, out = keep[li]
+        for (K, N, kind), (A, Q), xin, got, res in zip(shapes, layers[li], (x_in, o_in, f_in, d_in),
+                                                       (qkv, o, act, out), (None, None, None, x_in)):
+            qw, qz, sc = tm.unpack_repacked(A, Q, N, K, 128)
+            W = O.dequant_from_awq(host_u32(qw), host_u32(qz), sc.cpu().numpy(), 128)
+            want = O.epilogue(O.gemm_acc(xin, W), kind, res)
+            err = O.max_abs_rel(got, want)
+            assert err <= TOL, (li, K, N, kind, err)
+
+
 def test_errors(tm, gemm):
     T, K, N = 4, 256, 64
     d = O.make_inputs(1, T, K, N)
