@@ -31,6 +31,7 @@ MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16 matrix
 # HBM bytes per launch of the two dominant kernels, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
 # runs of `bench.py --probe ...`, calibrated against an elementwise kernel of known size
 # (profiles/decode_gate_up_hbm_traffic.md, profiles/prefill_gate_up_mfma_and_traffic.md).
+N_LAYERS = 32          # Llama-2-7B
 TRAFFIC_DECODE_GATE_UP = 49.36e6
 TRAFFIC_PREFILL_GATE_UP = 564.4e6
 
@@ -107,7 +108,7 @@ def main():
     weights = {}
     for name, K, N, epi in LAYER_7B:
         per_copy = K * N // 2 + (K // GROUP) * N * 4
-        n = max(args.copies, int(args.cold_gib * 2 ** 30 / per_copy) + 1)
+        n = max(args.copies, N_LAYERS, int(args.cold_gib * 2 ** 30 / per_copy) + 1)
         weights[name] = [make_weights(tm, torch, gen, name, K, N) for _ in range(n)]
     Tmax = max(max(DECODE_T), PREFILL_T)
     X = {K: torch.randn((Tmax, K), device="cuda", generator=gen).half() for K in (4096, 11008)}
@@ -241,6 +242,16 @@ def main():
                          "numpy unpack+dequantise %.2f s (1 thread) + torch fp32 matmul+epilogue %.3f s (%d threads)"
                          % (t_deq, t_mm, torch.get_num_threads())}
 
+    # ---- the full 32-layer GEMM sequence of one decode step at M = 8 (every layer its own weights) ----
+    seq_T = 8
+    seq_work = [[(name, layer, seq_T) for layer in range(N_LAYERS) for name, _, _, _ in LAYER_7B]]
+    seq_run = make_runner(seq_work)
+    seq_ms = timed(seq_run, 20, 5) / 20
+    seq_bytes = N_LAYERS * sum(algorithmic_bytes(seq_T, K, N, epi) for _, K, N, epi in LAYER_7B)
+    layers32 = {"T": seq_T, "layers": N_LAYERS, "gemms": 4 * N_LAYERS, "ms_per_decode_step": round(seq_ms, 4),
+                "GBps": round(seq_bytes / seq_ms / 1e6, 1), "frac": round(seq_bytes / seq_ms / 1e6 / HBM_PEAK_GBS, 4),
+                "weights_GB": round(N_LAYERS * sum(K * N // 2 + K // GROUP * N * 4 for _, K, N, _ in LAYER_7B) / 1e9, 2)}
+
     line = {
         "metric": "W4A16 GEMM achieved HBM GB/s (M=1..16) + TFLOP/s (M=2048), % of roofline",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -253,6 +264,7 @@ def main():
                    "bytes_per_step": step_bytes},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "roofline": roofline, "cpu_baseline": cpu, "decode_per_shape": per_shape, "prefill": prefill,
+        "layers32_m8": layers32,
     }
     print(json.dumps(line))
 
