@@ -218,6 +218,40 @@ def main():
                                 "traffic": TRAFFIC_PREFILL_GATE_UP if dom["shape"] == "gate_up" else None,
                                 "kernel": "prefill_kernel, %s, T=2048" % dom["shape"]}}
 
+    # ---- what this machine reaches with library kernels (context for the two peaks) ------------
+    # a device copy (read + write) for HBM, and hipBLASLt's fp16 GEMM on dense fp16 weights of the
+    # gate_up shape at T = 2048 (what the reference's non-quantised LlamaLinear path would call)
+    ceilings = None
+    if not args.no_prefill:
+        with torch.cuda.stream(stream):
+            src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
+            dst = torch.empty_like(src)
+            dst.copy_(src)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record(stream)
+            for _ in range(10):
+                dst.copy_(src)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            copy_gbs = 10 * 2 * src.numel() / e0.elapsed_time(e1) / 1e6
+            del src, dst
+            K, N = 4096, 22016
+            Wd = [torch.randn((K, N), device="cuda", generator=gen).half() for _ in range(4)]
+            Y = torch.empty((PREFILL_T, N), dtype=torch.float16, device="cuda")
+            torch.matmul(X[K][:PREFILL_T], Wd[0], out=Y)
+            torch.cuda.synchronize()
+            e0.record(stream)
+            for i in range(12):
+                torch.matmul(X[K][:PREFILL_T], Wd[i % 4], out=Y)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            dense_tf = 12 * flops(PREFILL_T, K, N) / e0.elapsed_time(e1) / 1e9
+            del Wd, Y
+        ceilings = {"device_copy_512MiB_GBps": round(copy_gbs, 1),
+                    "dense_fp16_gemm_gate_up_T2048_TFLOPs": round(dense_tf, 1),
+                    "note": "torch copy_ (bytes read + written) and torch.matmul fp16 (hipBLASLt) on this GPU"}
+
     # ---- CPU baseline: the oracle on the host cores, one layer at T = 8 -------------------------
     cpu = None
     if not args.no_cpu:
@@ -264,7 +298,7 @@ def main():
                    "bytes_per_step": step_bytes},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "roofline": roofline, "cpu_baseline": cpu, "decode_per_shape": per_shape, "prefill": prefill,
-        "layers32_m8": layers32,
+        "layers32_m8": layers32, "library_ceilings": ceilings,
     }
     print(json.dumps(line))
 
