@@ -79,10 +79,21 @@ int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const voi
 
 /* GemmS4F16::Measure (gemm_s4_f16.h:29-39, gemm_s4_f16.cu:98-169): times every feasible
  * kernel (10 warm-up + 100 timed launches each) and writes up to `capacity` rows sorted
- * by time; returns the number of rows, or a negative error.  Synchronises `stream`. */
+ * by time; returns the number of rows, or a negative error.  Synchronises `stream`.  The handle
+ * remembers the fastest kernel for (n_out, tokens, k); later `w4a16_gemm` calls with algo_id < 0
+ * and exactly that shape use it (see `w4a16_pick`). */
 int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R,
                   int n_out, int tokens, int k, int group_size, int epilogue,
                   w4a16_metric* metrics, int capacity, void* stream);
+
+/* The algo_id that `w4a16_gemm(..., algo_id = -1, ...)` would use for this shape: the fastest one a
+ * previous `w4a16_measure` on this handle found for exactly (n_out, tokens, k), else the heuristic's
+ * choice.  The reference's Measure only reports (gemm_s4_f16.cu:98-169) and its Run always
+ * estimates (gemm_s4_f16.cu:171-182); remembering the measurement is an extension.  Host-only. */
+int w4a16_pick(const w4a16_handle* h, int n_out, int tokens, int k);
+
+/* Forgets every measurement remembered by `w4a16_measure` on this handle. */
+int w4a16_clear_tuning(w4a16_handle* h);
 
 /* Number of kernels `w4a16_gemm` can dispatch to (valid algo_id are 0 .. count-1). */
 int w4a16_algo_count(void);

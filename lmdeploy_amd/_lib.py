@@ -39,6 +39,8 @@ SIGNATURES = {
     "w4a16_gemm": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_void_p]),
     "w4a16_measure": (c_int, [c_void_p] * 6 + [c_int] * 5 + [POINTER(Metric), c_int, c_void_p]),
     "w4a16_algo_count": (c_int, []),
+    "w4a16_pick": (c_int, [c_void_p, c_int, c_int, c_int]),
+    "w4a16_clear_tuning": (c_int, [c_void_p]),
     "w4a16_convert_s4_k_m8": (c_int, [c_void_p] * 6 + [c_int] * 3 + [c_void_p]),
     "w4a16_reformat_s4_k_m8": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "w4a16_fuse_w1_w3_s4_k_m8": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),

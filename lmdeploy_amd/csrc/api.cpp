@@ -9,6 +9,8 @@
 #include <cstdio>
 #include <cstring>
 #include <limits>
+#include <map>
+#include <tuple>
 #include <vector>
 
 namespace {
@@ -41,6 +43,8 @@ struct w4a16_handle {
     hipEvent_t     ev_end{};
     int            device{};
     w4a16::Scratch scratch{};
+    // fastest kernel found by w4a16_measure, per (n_out, tokens, k); consulted before the heuristic
+    std::map<std::tuple<int, int, int>, int> tuned;
 };
 
 namespace {
@@ -122,35 +126,47 @@ hipError_t algo_launch(int id, const GemmArgs& g, const Scratch& sc, hipStream_t
 int algo_pick(int N, int T, int K)
 {
     if (T <= 0 || N <= 0 || K <= 0) return -1;
-    if (T >= 64) {
-        // 128 x 128 tiles (two workgroups per CU) and 128 x 256 tiles (one per CU, half the LDS and
-        // L2 traffic per flop) run at about the same rate per CU; the wider tile wins when its
-        // workgroups fill the 256 CUs evenly (last round empty or more than 3/4 full), the narrower
-        // one otherwise because two small workgroups share a CU in the last round.  Narrower token
-        // tiles for short prompts.
-        bool wide = false;
-        if (N % 256 == 0 && T > 64) {
-            const int64_t wgs = (int64_t)(N / 256) * ((T + 127) / 128);
-            const int     rem = (int)(wgs % 256);
-            wide              = rem == 0 || rem > 192;
+    auto find_prefill = [&](int tile_t, int tile_n) {
+        for (int id = 0; id < algo_count(); ++id) {
+            const Algo& a = algo_at(id);
+            if (a.kind == 1 && a.tile_t == tile_t && a.tile_n == tile_n && algo_feasible(id, N, T, K)) return id;
         }
-        const int order[5][2] = {{128, wide ? 256 : 128}, {128, wide ? 128 : 256}, {64, 128}, {64, 64}, {256, 128}};  // tokens, features
-        for (auto& o : order) {
-            if (T <= 64 && o[0] > 64) continue;
-            for (int id = 0; id < algo_count(); ++id) {
-                const Algo& a = algo_at(id);
-                if (a.kind == 1 && a.tile_t == o[0] && a.tile_n == o[1] && algo_feasible(id, N, T, K)) return id;
-            }
+        return -1;
+    };
+    if (T > 32) {
+        // Prefill tiles by a cost model fitted to sweeps on MI355X: a CU works through its
+        // workgroups at a fixed rate per output element, so time ~ (workgroups / 256) x tile
+        // area x a penalty for small tiles (more dequantisation and LDS traffic per MFMA).  One
+        // tile's trip through K is the floor however idle the chip is, which is why short prompts
+        // want small tiles; ties go to the wider tile (less activation traffic).  If even the best
+        // tiling leaves more than a third of the CUs empty at <= 128 tokens (narrow matrices such as o_proj
+        // and down_proj) the decode kernels are faster.
+        struct Tile { int t, n; double penalty; };
+        const Tile tiles[5] = {{128, 256, 1.0}, {128, 128, 1.0}, {256, 128, 1.07}, {64, 128, 1.2}, {64, 64, 1.6}};
+        int    best = -1;
+        double best_cost = 0;
+        int64_t best_wgs = 0;
+        for (const Tile& t : tiles) {
+            if (N % t.n != 0) continue;
+            const int id = find_prefill(t.t, t.n);
+            if (id < 0) continue;
+            const int64_t wgs  = (int64_t)(N / t.n) * ((T + t.t - 1) / t.t);
+            // tiles with one workgroup per CU go in whole rounds; smaller ones share CUs, which evens out
+            const bool    one_per_cu = t.t * t.n > 128 * 128;
+            const double  rounds     = one_per_cu ? (double)((wgs + 255) / 256) : std::max(1.0, wgs / 256.0);
+            const double  cost       = rounds * t.t * t.n * t.penalty;
+            if (best < 0 || cost < best_cost * 0.999) best = id, best_cost = cost, best_wgs = wgs;
         }
-        for (int id = 0; id < algo_count(); ++id)
-            if (algo_at(id).kind == 1 && algo_feasible(id, N, T, K)) return id;
+        if (best >= 0 && (T > 128 || best_wgs >= 160) && (T >= 64 || best_wgs >= 256)) return best;
     }
     // Decode.  Strips of column tiles over the whole of K, one per CU, were the fastest on every
     // Llama-7B/70B shape measured at 1..16 tokens; two narrower strips per CU are slightly ahead on
     // very wide matrices while the activations are small.  Matrices with too few column tiles to
     // give every CU a strip fall back to the column-block kernel, which can also split K across
     // workgroups.
-    if (N / 16 >= 128) {
+    // Above 16 tokens every workgroup re-reads the weights once per 16-token block, and narrow
+    // matrices are better off splitting K across workgroups (column-block kernel with `fill`).
+    if (N / 16 >= 128 && (T <= 16 || N / 16 >= 512)) {
         const int want = (N / 16 >= 1024 && T <= 8) ? 2 : 1;
         for (int per_cu : {want, 1}) {
             for (int id = 0; id < algo_count(); ++id) {
@@ -213,6 +229,14 @@ int check_gemm_args(const w4a16_handle* h, const void* C, const void* A, const v
     return 0;
 }
 
+// the kernel w4a16_gemm uses for algo_id < 0: a measured one if this exact shape was measured
+int pick_for(const w4a16_handle* h, int n_out, int tokens, int k)
+{
+    const auto it = h->tuned.find(std::make_tuple(n_out, tokens, k));
+    if (it != h->tuned.end() && algo_feasible(it->second, n_out, tokens, k)) return it->second;
+    return algo_pick(n_out, tokens, k);
+}
+
 }  // namespace
 
 extern "C" {
@@ -253,6 +277,22 @@ void w4a16_destroy(w4a16_handle* h)
     delete h;
 }
 
+int w4a16_pick(const w4a16_handle* h, int n_out, int tokens, int k)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    if (n_out <= 0 || tokens <= 0 || k <= 0 || k % 128 != 0 || n_out % 16 != 0)
+        return fail(W4A16_ESHAPE, "no feasible kernel found");
+    const int id = pick_for(h, n_out, tokens, k);
+    return id >= 0 ? id : fail(W4A16_ESHAPE, "no feasible kernel found");
+}
+
+int w4a16_clear_tuning(w4a16_handle* h)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    h->tuned.clear();
+    return W4A16_OK;
+}
+
 int w4a16_algo_count(void)
 {
     return algo_count();
@@ -265,7 +305,7 @@ int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const voi
     if (chk < 0) return chk;
     if (chk > 0) return W4A16_OK;
     if (algo_id >= algo_count()) return fail(W4A16_EALGO, "algo_id %d out of range (0..%d)", algo_id, algo_count() - 1);
-    if (algo_id < 0) algo_id = algo_pick(n_out, tokens, k);
+    if (algo_id < 0) algo_id = pick_for(h, n_out, tokens, k);
     if (algo_id < 0 || !algo_feasible(algo_id, n_out, tokens, k)) return fail(W4A16_ESHAPE, "no feasible kernel found");
     GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
                n_out,        tokens,             k,                  epilogue};
@@ -283,7 +323,7 @@ int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const 
     if (chk > 0) return 0;
     constexpr int kWarmup = 10, kMeasure = 100;  // gemm_s4_f16.cu:258-259
     hipStream_t   st   = (hipStream_t)stream;
-    const int     best = algo_pick(n_out, tokens, k);
+    const int     best = pick_for(h, n_out, tokens, k);
     GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
                n_out,        tokens,             k,                  epilogue};
     std::vector<w4a16_metric> all;
@@ -318,6 +358,7 @@ int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const 
         all.push_back(m);
     }
     std::stable_sort(all.begin(), all.end(), [](const w4a16_metric& a, const w4a16_metric& b) { return a.ms < b.ms; });
+    if (!all.empty() && all.front().feasible) h->tuned[std::make_tuple(n_out, tokens, k)] = all.front().id;
     const int n = std::min<int>(capacity, (int)all.size());
     std::memcpy(metrics, all.data(), sizeof(w4a16_metric) * n);
     return n;

@@ -124,3 +124,11 @@ class GemmS4F16:
     @staticmethod
     def algo_count() -> int:
         return lib.w4a16_algo_count()
+
+    def pick(self, m: int, n: int, k: int) -> int:
+        """The algo_id that `Run(..., algo_id=-1)` uses for this shape: the fastest one a previous
+        `Measure` of exactly this shape found, else the heuristic's choice."""
+        return check(lib.w4a16_pick(self._h, m, n, k))
+
+    def clear_tuning(self) -> None:
+        check(lib.w4a16_clear_tuning(self._h))

@@ -362,3 +362,13 @@ def test_measure_reports_all_kernels(tm, gemm):
     assert feas and all(np.isfinite(m.ms) and m.count == 100 for m in feas)
     assert [m.ms for m in ms] == sorted(m.ms for m in ms)
     assert sum(m.best for m in ms) == 1
+    # the handle remembers the winner for exactly this shape and Run(algo_id=-1) uses it
+    assert gemm.pick(N, T, K) == ms[0].id
+    got = run(tm, gemm, d, A, Q, T, K, N, 0)
+    assert O.max_abs_rel(got, O.gemm_s4_f16(d["X"], d["qweight"], d["qzeros"], d["scales"], 128)) <= TOL
+    other = tm.GemmS4F16()                      # a fresh handle knows nothing: heuristic choice
+    heuristic = other.pick(N, T, K)
+    gemm.clear_tuning()
+    assert gemm.pick(N, T, K) == heuristic
+    with pytest.raises(tm.W4A16Error):
+        gemm.pick(N + 8, T, K)
