@@ -152,7 +152,7 @@ int algo_pick(int N, int T, int K)
             if (id < 0) continue;
             const int64_t wgs  = (int64_t)(N / t.n) * ((T + t.t - 1) / t.t);
             // tiles with one workgroup per CU go in whole rounds; smaller ones share CUs, which evens out
-            const bool    one_per_cu = t.t * t.n > 128 * 128;
+            const bool    one_per_cu = t.t * t.n > 128 * 128;  // (also the eight-wave 128 x 256 tile: it fills a CU)
             const double  rounds     = one_per_cu ? (double)((wgs + 255) / 256) : std::max(1.0, wgs / 256.0);
             const double  cost       = rounds * t.t * t.n * t.penalty;
             if (best < 0 || cost < best_cost * 0.999) best = id, best_cost = cost, best_wgs = wgs;

@@ -1,6 +1,7 @@
 // Prefill W4A16 GEMM for gfx950: many tokens, bound by the fp16 MFMA rate.
 //
-// A workgroup of four waves computes a (16*TTILES tokens) x (64*NTW features) output tile.
+// A workgroup of four (or eight) waves computes a (16*TTILES tokens) x (16*NTW*WAVES features)
+// output tile.
 // The waves split the features; each owns NTW weight tiles per quantisation group and loads
 // them straight from global memory into registers (one 128-bit load per lane and tile: the
 // tiled layout IS the MFMA operand layout), dequantises them to the reference's exact fp16
@@ -27,7 +28,6 @@ namespace w4a16 {
 
 namespace {
 
-constexpr int kThreads   = 256;
 // LDS holds two activation tiles of [tokens][128 halves] = 256 bytes per token row, i.e. 16 chunks
 // of 16 bytes.  Chunk position p of row r holds K-chunk p ^ (r & 15): the 16 lanes that read the
 // same K-chunk of 16 consecutive rows then hit 16 different bank groups, without padding, which
@@ -86,15 +86,18 @@ __device__ __forceinline__ void wait_lgkm0(half8_t& a, half8_t& b, half8_t& c, h
 // VGPRs and parking values in AGPRs, which is fatal here: a register parked while an
 // inline-assembly load into it is still in flight is handed to another value, and the load then
 // lands on that value (the build rejects kernels that use AGPRs beyond their accumulators).
-template<int TTILES, int NTW, int EPI>
-__global__ void __launch_bounds__(kThreads)
+// WAVES = waves per workgroup (4 or 8), side by side along the features.
+template<int TTILES, int NTW, int WAVES, int EPI>
+__global__ void __launch_bounds__(64 * WAVES)
     __attribute__((amdgpu_waves_per_eu(TTILES * NTW >= 32 ? 1 : 2, TTILES * NTW >= 32 ? 1 : 2)))
 prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const uint16_t* __restrict__ X,
                const uint32_t* __restrict__ Q, const uint16_t* R_, int N, int T, int K, int tiles_t, int tiles_n)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [2][TT][kRowBytes]
     constexpr int TT = 16 * TTILES;
-    constexpr int TN = 64 * NTW;
+    constexpr int TN = 16 * NTW * WAVES;
+    constexpr int XB = 4 * TTILES / WAVES;  // 1 KiB activation blocks (4 token rows) that each wave fetches per group
+    static_assert(4 * TTILES % WAVES == 0, "the activation tile must divide evenly among the waves");
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
@@ -128,14 +131,14 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     // per-thread byte offsets; the group-dependent part of every address is scalar
     const uint32_t w_off = (uint32_t)(nt0 * 1024 + lane * 16);        // + g * NT * 1024 (+ nt * 1024)
     const uint32_t q_off = (uint32_t)((nt0 * kTileN + c) * 4);        // + g * N * 4    (+ nt * 64)
-    // X staging, direct global -> LDS: wave w, request i writes the 1 KiB block m = w*TTILES + i
+    // X staging, direct global -> LDS: wave w, request i writes the 1 KiB block m = w*XB + i
     // (token rows 4m .. 4m+3) of the tile; lane l lands at row 4m + l/16, chunk position l%16, so it
     // fetches K-chunk (l%16) ^ (row & 15) of that row.  Rows past the last token re-read the last
     // valid row; their outputs are never stored.
-    uint32_t x_off[TTILES];
+    uint32_t x_off[XB];
 #pragma unroll
-    for (int i = 0; i < TTILES; ++i) {
-        const int row = 4 * (wave * TTILES + i) + (lane >> 4);
+    for (int i = 0; i < XB; ++i) {
+        const int row = 4 * (wave * XB + i) + (lane >> 4);
         x_off[i] = (uint32_t)min(T0 + row, T - 1) * (uint32_t)(K * 2) + (uint32_t)(((lane & 15) ^ (row & 15)) * 16);
     }
     // fragment reads: lane (c, b) reads row 16*tt + c, K-chunk 4j + b  ->  position (4j + b) ^ c
@@ -169,14 +172,14 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     auto issue_x = [&](uint8_t* xo, int g) {
         const char* xbase = reinterpret_cast<const char*>(X) + (int64_t)g * 256;
 #pragma unroll
-        for (int i = 0; i < TTILES; ++i) {
+        for (int i = 0; i < XB; ++i) {
             __builtin_amdgcn_global_load_lds(
                 (const __attribute__((address_space(1))) void*)(xbase + x_off[i]),
-                (__attribute__((address_space(3))) void*)(xo + (wave * TTILES + i) * 1024), 16, 0, 0);
+                (__attribute__((address_space(3))) void*)(xo + (wave * XB + i) * 1024), 16, 0, 0);
         }
     };
     // the same requests one at a time (m = 0 .. 2 NTW + TTILES - 1), to be dealt out between MFMAs
-    constexpr int kVmOps = 2 * NTW + TTILES;
+    constexpr int kVmOps = 2 * NTW + XB;
     auto vm_op = [&](auto M, u32x4_t (&w)[NTW], uint32_t (&qv)[NTW], uint8_t* xo, const char* wbase, const char* qbase,
                      const char* xbase) {
         constexpr int m = decltype(M)::value;
@@ -190,7 +193,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
             constexpr int i = m - 2 * NTW;
             __builtin_amdgcn_global_load_lds(
                 (const __attribute__((address_space(1))) void*)(xbase + x_off[i]),
-                (__attribute__((address_space(3))) void*)(xo + (wave * TTILES + i) * 1024), 16, 0, 0);
+                (__attribute__((address_space(3))) void*)(xo + (wave * XB + i) * 1024), 16, 0, 0);
         }
     };
     auto wait_all = [&](u32x4_t (&w)[NTW], uint32_t (&qv)[NTW]) {
@@ -373,25 +376,26 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
 }
 
 struct Variant {
-    int ttiles, ntw;
+    int ttiles, ntw, waves;
 };
 // (a 256 x 256 tile does not fit the register file without spilling, and spill stores would
 // break the counted waits: stores and loads complete out of order with each other)
-constexpr Variant kVariants[] = {{8, 4}, {16, 2}, {8, 2}, {4, 2}, {4, 1}};
+// (first match wins in the dispatcher: the 8-wave 128 x 256 tile comes before the 4-wave one)
+constexpr Variant kVariants[] = {{8, 2, 8}, {16, 2, 4}, {8, 2, 4}, {4, 2, 4}, {4, 1, 4}, {8, 4, 4}};
 constexpr int     kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
-template<int TTILES, int NTW>
+template<int TTILES, int NTW, int WAVES>
 hipError_t launch_v(const GemmArgs& a, hipStream_t st)
 {
-    constexpr int TT = 16 * TTILES, TN = 64 * NTW;
+    constexpr int TT = 16 * TTILES, TN = 16 * NTW * WAVES;
     const int     tiles_t = (a.T + TT - 1) / TT;
     const int     tiles_n = a.N / TN;
     const size_t  lds     = (size_t)2 * TT * kRowBytes;
-    const dim3    grid(tiles_t * tiles_n), block(kThreads);
+    const dim3    grid(tiles_t * tiles_n), block(64 * WAVES);
     const u32x4_t* A4 = reinterpret_cast<const u32x4_t*>(a.A);
 #define W4A16_LAUNCH(EPI)                                                                                              \
     do {                                                                                                               \
-        auto       kfn = prefill_kernel<TTILES, NTW, EPI>;                                                             \
+        auto       kfn = prefill_kernel<TTILES, NTW, WAVES, EPI>;                                                             \
         hipError_t e   = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),                                       \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
         if (e != hipSuccess) return e;                                                                                 \
@@ -415,14 +419,14 @@ int prefill_variants()
 
 void prefill_tile(int v, int& tile_n, int& tile_t)
 {
-    tile_n = 64 * kVariants[v].ntw;
+    tile_n = 16 * kVariants[v].ntw * kVariants[v].waves;
     tile_t = 16 * kVariants[v].ttiles;
 }
 
 bool prefill_feasible(int v, int N, int T, int K)
 {
     if (v < 0 || v >= kNumVariants || N <= 0 || T <= 0 || K <= 0) return false;
-    const int tn = 64 * kVariants[v].ntw, tt = 16 * kVariants[v].ttiles;
+    const int tn = 16 * kVariants[v].ntw * kVariants[v].waves, tt = 16 * kVariants[v].ttiles;
     if (N % tn != 0 || K % kGroup != 0) return false;
     // per-thread offsets into X and into one group of A are 32-bit
     if ((int64_t)T * K * 2 >= (1ll << 32) || (int64_t)N * 64 >= (1ll << 32)) return false;
@@ -433,18 +437,19 @@ bool prefill_feasible(int v, int N, int T, int K)
 int prefill_grid(int v, int N, int T, int K)
 {
     (void)K;
-    const int tn = 64 * kVariants[v].ntw, tt = 16 * kVariants[v].ttiles;
+    const int tn = 16 * kVariants[v].ntw * kVariants[v].waves, tt = 16 * kVariants[v].ttiles;
     return (N / tn) * ((T + tt - 1) / tt);
 }
 
 hipError_t prefill_launch(int v, const GemmArgs& a, hipStream_t st)
 {
     switch (v) {
-        case 0: return launch_v<8, 4>(a, st);
-        case 1: return launch_v<16, 2>(a, st);
-        case 2: return launch_v<8, 2>(a, st);
-        case 3: return launch_v<4, 2>(a, st);
-        default: return launch_v<4, 1>(a, st);
+        case 0: return launch_v<8, 2, 8>(a, st);
+        case 1: return launch_v<16, 2, 4>(a, st);
+        case 2: return launch_v<8, 2, 4>(a, st);
+        case 3: return launch_v<4, 2, 4>(a, st);
+        case 4: return launch_v<4, 1, 4>(a, st);
+        default: return launch_v<8, 4, 4>(a, st);
     }
 }
 
