@@ -257,24 +257,28 @@ def main():
     if not args.no_cpu:
         import numpy as np
         from oracle import w4a16_oracle as O
-        T = 8
+        T, reps = 8, 5
         t_deq = t_mm = 0.0
         by = 0
         for i, (name, K, N, epi) in enumerate(LAYER_7B):
             d = O.make_inputs(77 + i, T, K, N, GROUP, residual=(epi == 2))
-            t0 = time.perf_counter()
-            W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], GROUP)
-            t1 = time.perf_counter()
-            O.epilogue(O.gemm_acc(d["X"], W), epi, d.get("R"))
-            t2 = time.perf_counter()
-            t_deq += t1 - t0
-            t_mm += t2 - t1
+            deq, mm = [], []
+            for _ in range(reps):   # median of five passes per GEMM, both halves timed separately
+                t0 = time.perf_counter()
+                W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], GROUP)
+                t1 = time.perf_counter()
+                O.epilogue(O.gemm_acc(d["X"], W), epi, d.get("R"))
+                t2 = time.perf_counter()
+                deq.append(t1 - t0)
+                mm.append(t2 - t1)
+            t_deq += sorted(deq)[reps // 2]
+            t_mm += sorted(mm)[reps // 2]
             by += algorithmic_bytes(T, K, N, epi)
         cpu = {"value": round(by / (t_deq + t_mm) / 1e9, 4), "unit": "GB/s", "cores": torch.get_num_threads(),
                "kind": "port", "host_cpus": os.cpu_count(),
-               "sample": "one Llama-2-7B layer (qkv, o, gate_up+SiLU, down+residual) at T=8, single pass: "
-                         "numpy unpack+dequantise %.2f s (1 thread) + torch fp32 matmul+epilogue %.3f s (%d threads)"
-                         % (t_deq, t_mm, torch.get_num_threads())}
+               "sample": "one Llama-2-7B layer (qkv, o, gate_up+SiLU, down+residual) at T=8, median of %d passes per "
+                         "GEMM: numpy unpack+dequantise %.2f s (1 thread) + torch fp32 matmul+epilogue %.3f s "
+                         "(%d threads)" % (reps, t_deq, t_mm, torch.get_num_threads())}
 
     # ---- the full 32-layer GEMM sequence of one decode step at M = 8 (every layer its own weights) ----
     seq_T = 8

@@ -77,6 +77,17 @@ void w4a16_destroy(w4a16_handle* h);
 int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R,
                int n_out, int tokens, int k, int group_size, int epilogue, int algo_id, void* stream);
 
+/* The int4 branch of LlamaFfnLayer<T>::forward (src/turbomind/models/llama/LlamaFfnLayer.cc:67-116)
+ * as one call: gating = SiLU-gated fused gate/up GEMM (kFusedSiluFfn) into `gating_buf`
+ * [tokens, inter_size], then ffn_output = gating * W2 (+ residual if `residual` is not null: the add
+ * half of the fused add-norm that follows in LlamaDecoder.cc:228-235; `residual` may alias
+ * `ffn_output`).  A13/Q13 are the converted fused w1|w3 weights (n_out = 2 * inter_size, k =
+ * hidden_units), A2/Q2 the converted w2 (n_out = hidden_units, k = inter_size).  Both launches go to
+ * `stream` back to back; nothing is allocated, so the call can be captured in a HIP graph. */
+int w4a16_ffn(w4a16_handle* h, void* ffn_output, void* gating_buf, const void* ffn_input, const void* A13,
+              const void* Q13, const void* A2, const void* Q2, const void* residual, int hidden_units,
+              int inter_size, int tokens, int group_size, void* stream);
+
 /* GemmS4F16::Measure (gemm_s4_f16.h:29-39, gemm_s4_f16.cu:98-169): times every feasible
  * kernel (10 warm-up + 100 timed launches each) and writes up to `capacity` rows sorted
  * by time; returns the number of rows, or a negative error.  Synchronises `stream`.  The handle

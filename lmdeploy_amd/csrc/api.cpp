@@ -314,6 +314,18 @@ int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const voi
     return W4A16_OK;
 }
 
+int w4a16_ffn(w4a16_handle* h, void* ffn_output, void* gating_buf, const void* ffn_input, const void* A13,
+              const void* Q13, const void* A2, const void* Q2, const void* residual, int hidden_units,
+              int inter_size, int tokens, int group_size, void* stream)
+{
+    if (hidden_units < 0 || inter_size < 0) return fail(W4A16_EARG, "negative size");
+    const int rc = w4a16_gemm(h, gating_buf, A13, ffn_input, Q13, nullptr, 2 * inter_size, tokens, hidden_units,
+                              group_size, W4A16_FUSED_SILU_FFN, -1, stream);
+    if (rc != W4A16_OK) return rc;
+    return w4a16_gemm(h, ffn_output, A2, gating_buf, Q2, residual, hidden_units, tokens, inter_size, group_size,
+                      residual ? W4A16_FUSED_ADD : W4A16_GEMM, -1, stream);
+}
+
 int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R, int n_out,
                   int tokens, int k, int group_size, int epilogue, w4a16_metric* metrics, int capacity, void* stream)
 {

@@ -125,6 +125,15 @@ class GemmS4F16:
     def algo_count() -> int:
         return lib.w4a16_algo_count()
 
+    def ffn(self, ffn_output, gating_buf, ffn_input, A13, Q13, A2, Q2, hidden_units: int, inter_size: int, n: int,
+            group_size: int = 128, residual=None, stream: Optional[int] = None) -> None:
+        """The int4 branch of LlamaFfnLayer<T>::forward (LlamaFfnLayer.cc:67-116): SiLU-gated fused
+        gate/up GEMM into `gating_buf` [n, inter_size], then w2 into `ffn_output` [n, hidden_units],
+        plus `residual` if given (may alias `ffn_output`)."""
+        check(lib.w4a16_ffn(self._h, _ptr(ffn_output), _ptr(gating_buf), _ptr(ffn_input), _ptr(A13), _ptr(Q13),
+                            _ptr(A2), _ptr(Q2), _ptr(residual), hidden_units, inter_size, n, group_size,
+                            _stream() if stream is None else stream))
+
     def pick(self, m: int, n: int, k: int) -> int:
         """The algo_id that `Run(..., algo_id=-1)` uses for this shape: the fastest one a previous
         `Measure` of exactly this shape found, else the heuristic's choice."""

@@ -330,6 +330,33 @@ def test_llama7b_32_layer_decode_sequence(tm, gemm):
             assert err <= TOL, (li, K, N, kind, err)
 
 
+def test_ffn_block(tm, gemm):
+    """LlamaFfnLayer's int4 branch as one call: fused gate/up + SiLU into the gating buffer, then w2
+    (+ residual, in place), against the oracle chained through the same fp16 intermediate."""
+    T, H, F = 6, 512, 768
+    d13 = O.make_inputs(31, T, H, 2 * F)
+    d2 = O.make_inputs(32, T, F, H, residual=True)
+    A13, Q13 = convert(tm, d13, 2 * F, H)
+    A2, Q2 = convert(tm, d2, H, F)
+    x = dev(d13["X"])
+    gating = torch.empty((T, F), dtype=torch.float16, device="cuda")
+    out = torch.empty((T, H), dtype=torch.float16, device="cuda")
+    gemm.ffn(out, gating, x, A13, Q13, A2, Q2, H, F, T)
+    torch.cuda.synchronize()
+    want_g = O.gemm_s4_f16(d13["X"], d13["qweight"], d13["qzeros"], d13["scales"], 128, O.EPI_SILU)
+    assert O.max_abs_rel(gating.cpu().numpy(), want_g) <= TOL
+    g_host = gating.cpu().numpy()               # the second GEMM is checked on the GPU's own intermediate
+    want = O.gemm_s4_f16(g_host, d2["qweight"], d2["qzeros"], d2["scales"], 128)
+    assert O.max_abs_rel(out.cpu().numpy(), want) <= TOL
+    res = dev(d2["R"])
+    gemm.ffn(res, gating, x, A13, Q13, A2, Q2, H, F, T, residual=res)     # output aliases the residual
+    torch.cuda.synchronize()
+    want = O.gemm_s4_f16(g_host, d2["qweight"], d2["qzeros"], d2["scales"], 128, O.EPI_ADD, d2["R"])
+    assert O.max_abs_rel(res.cpu().numpy(), want) <= TOL
+    with pytest.raises(tm.W4A16Error):
+        gemm.ffn(out, gating, x, A13, Q13, A2, Q2, H, F, T, group_size=64)
+
+
 def test_errors(tm, gemm):
     T, K, N = 4, 256, 64
     d = O.make_inputs(1, T, K, N)
