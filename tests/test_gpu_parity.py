@@ -330,6 +330,23 @@ def test_llama7b_32_layer_decode_sequence(tm, gemm):
             assert err <= TOL, (li, K, N, kind, err)
 
 
+@pytest.mark.parametrize("K,N", [(1024, 3072), (512, 4112), (128, 16), (2048, 2064)])
+def test_default_dispatch_over_token_counts(tm, gemm, K, N):
+    """`algo_id = -1` across the hand-over points between the decode, strip and prefill kernels,
+    on shapes with and without the divisibility the wider tiles need (4112 = 16 * 257, 2064 = 16 * 129)."""
+    Ts = (1, 5, 16, 17, 33, 48, 64, 100, 129, 192, 300, 1000)
+    d = O.make_inputs(900 + K + N, max(Ts), K, N, residual=True)
+    A, Q = convert(tm, d, N, K)
+    W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], 128)
+    for kind in ((0, 2) if N % 32 else (0, 1, 2)):
+        for T in Ts:
+            dd = dict(d, X=d["X"][:T], R=d["R"][:T])
+            want = O.epilogue(O.gemm_acc(dd["X"], W), kind, dd["R"] if kind == 2 else None)
+            got = run(tm, gemm, dd, A, Q, T, K, N, kind)
+            err = O.max_abs_rel(got, want)
+            assert np.isfinite(got).all() and err <= TOL, (K, N, kind, T, gemm.pick(N, T, K), err)
+
+
 def test_ffn_block(tm, gemm):
     """LlamaFfnLayer's int4 branch as one call: fused gate/up + SiLU into the gating buffer, then w2
     (+ residual, in place), against the oracle chained through the same fp16 intermediate."""
