@@ -85,23 +85,8 @@ __device__ __forceinline__ void unpack_offset(uint32_t w, uint32_t (&v)[4], cons
     v[3] = (w8 & k.mask_hi) | k.magic_hi;
 }
 
-// One weight word -> eight fp16 values (q - z), rows 0..7 in order.  z1024 = (1024 + z) x2 and
-// z64 = (64 + z) x2; both subtractions are exact.
-__device__ __forceinline__ half8_t dequant_sub(uint32_t w, half2_t z1024, half2_t z64, const UnpackConsts& k)
-{
-    uint32_t v[4];
-    unpack_offset(w, v, k);
-    const half2_t a = as_half2(v[0]) - z1024;
-    const half2_t b = as_half2(v[1]) - z64;
-    const half2_t c = as_half2(v[2]) - z1024;
-    const half2_t d = as_half2(v[3]) - z64;
-    half8_t r;
-    r[0] = a[0]; r[1] = a[1]; r[2] = b[0]; r[3] = b[1];
-    r[4] = c[0]; r[5] = c[1]; r[6] = d[0]; r[7] = d[1];
-    return r;
-}
-
-// Same, then multiplied by the scale in fp16: fp16_rn((q - z) * s), the reference's weight.
+// One weight word -> eight fp16 weights, rows 0..7 in order: fp16_rn((q - z) * s), the reference's
+// weight.  z1024 = (1024 + z) x2 and z64 = (64 + z) x2; both subtractions are exact.
 __device__ __forceinline__ half8_t dequant_full(uint32_t w, half2_t z1024, half2_t z64, half2_t s,
                                                 const UnpackConsts& k)
 {
