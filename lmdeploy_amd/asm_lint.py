@@ -8,6 +8,17 @@ control-flow graph of every kernel, propagates "VGPR v is the destination of the
 load in flight" to a fixed point (a wait for vmcnt(N) retires every load with p > N; where paths
 join, the younger position wins), and reports any compiler-generated instruction that touches a
 register whose load may still be in flight.
+
+LDS reads issued from inline assembly (`ds_read_*`) are tracked the same way, more coarsely: their
+destinations stay in flight until a wait for lgkmcnt(0).  (A destination that nothing reads any
+more is the dangerous one: the compiler hands the register to another value at once, and the
+read lands on it later.)
+
+MFMAs issued from inline assembly hide a third hazard: the hardware does not interlock a matrix
+instruction's result against vector instructions, the compiler normally pads with s_nop, and it
+cannot see into inline assembly.  Compiler-generated accumulator moves (`v_accvgpr_*`) must
+therefore not follow an inline-assembly MFMA that writes the same AGPR within `_MFMA_SETTLE` wait
+states, nor write an AGPR that an inline-assembly MFMA reads within the next two.
 """
 from __future__ import annotations
 
@@ -15,6 +26,7 @@ import re
 from typing import Dict, List, Tuple
 
 _LOAD = re.compile(r"^\s*global_load_(?:lds_)?dword(?:x2|x3|x4)?\s+v(?:\[(\d+):(\d+)\]|(\d+))\s*,")
+_DSREAD = re.compile(r"^\s*ds_read\w*\s+v(?:\[(\d+):(\d+)\]|(\d+))\s*,")
 _STORE = re.compile(r"^\s*global_(?:store|atomic)\w*\s")
 _VMCNT = re.compile(r"vmcnt\((\d+)\)")
 _VREG = re.compile(r"\bv(?:\[(\d+):(\d+)\]|(\d+))\b")
@@ -79,12 +91,18 @@ def _parse(lines: List[Tuple[int, str]]):
         if _STORE.match(code):
             cur.append(_Ins("load", [], 0, code, ln))  # stores count in vmcnt too: only makes waits conservative
             continue
+        if in_asm:
+            m = _DSREAD.match(code)
+            if m:
+                cur.append(_Ins("ldsread", list(_regs(m)), 0, code, ln))
+                continue
         if code.startswith("s_waitcnt"):
+            everything = re.match(r"s_waitcnt\s+(0|0x0)\s*$", code) is not None
             v = _VMCNT.search(code)
-            if v is not None:
-                cur.append(_Ins("wait", [], int(v.group(1)), code, ln))
-            elif re.match(r"s_waitcnt\s+(0|0x0)\s*$", code):
-                cur.append(_Ins("wait", [], 0, code, ln))
+            if v is not None or everything:
+                cur.append(_Ins("wait", [], 0 if everything else int(v.group(1)), code, ln))
+            if everything or "lgkmcnt(0)" in code:
+                cur.append(_Ins("ldswait", [], 0, code, ln))
             continue
         if in_asm:
             continue  # hand-written: assumed to respect the waits it places
@@ -97,20 +115,77 @@ def _parse(lines: List[Tuple[int, str]]):
 
 
 def _transfer(state: Dict[int, int], ins: List[_Ins], report=None) -> Dict[int, int]:
+    """state: register -> position of its load among those in flight (1 = youngest); a register
+    with an LDS read in flight is kept under the key -(register + 1)."""
     st = dict(state)
     for i in ins:
         if i.kind == "load":
-            st = {r: p + 1 for r, p in st.items()}
+            st = {r: (p + 1 if r >= 0 else p) for r, p in st.items()}
             for r in i.regs:
                 st[r] = 1
         elif i.kind == "wait":
-            st = {r: p for r, p in st.items() if p <= i.n}
+            st = {r: p for r, p in st.items() if r < 0 or p <= i.n}
+        elif i.kind == "ldsread":
+            for r in i.regs:
+                st[-(r + 1)] = 0
+        elif i.kind == "ldswait":
+            st = {r: p for r, p in st.items() if r >= 0}
         elif report is not None:
             for r in i.regs:
-                if r in st:
+                if r in st or -(r + 1) in st:
                     report(i, r)
                     break
     return st
+
+
+_MFMA_SETTLE = 20  # wait states after which the result of the longest MFMA used here (8 passes) is readable
+_MFMA = re.compile(r"^\s*v_mfma\w*\s+a\[(\d+):(\d+)\]\s*,(.*)$")
+_AREG = re.compile(r"\ba(?:\[(\d+):(\d+)\]|(\d+))\b")
+_NOP = re.compile(r"^\s*s_nop\s+(\d+)")
+
+
+def _mfma_hazards(name: str, lines: List[Tuple[int, str]]) -> List[str]:
+    """Textual (fall-through order) check of compiler-generated AGPR moves next to inline-assembly MFMAs."""
+    seq, in_asm = [], False  # (line, code, in_asm)
+    for ln, raw in lines:
+        s = raw.strip()
+        if s.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if s.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        code = raw.split(";")[0].strip()
+        if not code or code.startswith(".") or code.endswith(":"):
+            continue
+        seq.append((ln, code, in_asm))
+    out = []
+    for k, (ln, code, asm) in enumerate(seq):
+        if asm or not code.startswith("v_accvgpr"):
+            continue
+        mine = {r for m in _AREG.finditer(code) for r in _regs(m)}
+        waited, j = 0, k - 1
+        while j >= 0 and waited < _MFMA_SETTLE:
+            pl, pc, pasm = seq[j]
+            if pc.startswith("s_branch") or pc.startswith("s_endpgm"):
+                break  # not reached from the text above
+            m = _MFMA.match(pc) if pasm else None
+            if m and mine & set(range(int(m.group(1)), int(m.group(2)) + 1)):
+                out.append("%s: line %d moves an accumulator %d wait states after the MFMA of line %d wrote it: %s"
+                           % (name, ln, waited, pl, code))
+                break
+            n = _NOP.match(pc)
+            waited += int(n.group(1)) + 1 if n else 1
+            j -= 1
+        if code.startswith("v_accvgpr_write") or code.startswith("v_accvgpr_mov"):
+            dst = next(iter(_regs(_AREG.search(code))))
+            for pl, pc, pasm in seq[k + 1:k + 3]:
+                m = _MFMA.match(pc) if pasm else None
+                if m and dst in {r for a in _AREG.finditer(m.group(3)) for r in _regs(a)}:
+                    out.append("%s: line %d writes a%d right before the MFMA of line %d reads it: %s"
+                               % (name, ln, dst, pl, code))
+                    break
+    return out
 
 
 def lint(asm_text: str, only_if_name_has: str = "kernel") -> List[str]:
@@ -130,6 +205,7 @@ def lint(asm_text: str, only_if_name_has: str = "kernel") -> List[str]:
         if name is not None:
             cur.append((ln, raw))
     for name, lines in funcs:
+        out.extend(_mfma_hazards(name, lines))
         blocks = _parse(lines)
         index = {b[0]: k for k, b in enumerate(blocks)}
         entry: List[Dict[int, int]] = [None] * len(blocks)  # type: ignore

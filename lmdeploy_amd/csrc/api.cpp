@@ -47,11 +47,6 @@ struct w4a16_handle {
     std::map<std::tuple<int, int, int>, int> tuned;
 };
 
-namespace {
-constexpr size_t kWorkspaceBytes = 64u << 20;  // split-K partial tiles
-constexpr int    kCounters       = 1 << 16;    // one per column block and token row block
-}  // namespace
-
 namespace w4a16 {
 
 // ---- kernel table (the counterpart of the 17 GemmKernel objects of gemm_s4_f16.cu:72-93) ----
@@ -76,6 +71,14 @@ std::vector<Algo> build_table()
         int tn = 0, tt = 0;
         prefill_tile(v, tn, tt);
         t.push_back(Algo{1, tn, tt, 1, v, DecodeConfig{}});
+    }
+    // the same tiles with K split across 2, 4 or 8 workgroups (few tokens: too few tiles to fill the chip)
+    for (int splits : {2, 4, 8}) {
+        for (int v = 0; v < prefill_variants(); ++v) {
+            int tn = 0, tt = 0;
+            prefill_tile(v, tn, tt);
+            if (tt <= 128) t.push_back(Algo{1, tn, tt, splits, v, DecodeConfig{}});
+        }
     }
     return t;
 }
@@ -102,14 +105,14 @@ bool algo_feasible(int id, int N, int T, int K)
 {
     const Algo& a = algo_at(id);
     if (a.kind == 2) return strip_feasible(a.param, N, T, K);
-    return a.kind == 0 ? decode_feasible(a.dc, N, T, K) : prefill_feasible(a.param, N, T, K);
+    return a.kind == 0 ? decode_feasible(a.dc, N, T, K) : prefill_feasible(a.param, a.slices, N, T, K);
 }
 
 int algo_grid(int id, int N, int T, int K, const Scratch& sc)
 {
     const Algo& a = algo_at(id);
     if (a.kind == 2) return strip_grid(a.param, N, T, K);
-    return a.kind == 0 ? decode_grid(a.dc, N, T, K, sc.ws_bytes, sc.cnt_len) : prefill_grid(a.param, N, T, K);
+    return a.kind == 0 ? decode_grid(a.dc, N, T, K, sc.ws_bytes, sc.cnt_len) : prefill_grid(a.param, a.slices, N, T, K);
 }
 
 hipError_t algo_launch(int id, const GemmArgs& g, const Scratch& sc, hipStream_t st)
@@ -117,7 +120,7 @@ hipError_t algo_launch(int id, const GemmArgs& g, const Scratch& sc, hipStream_t
     const Algo& a = algo_at(id);
     if (a.kind == 2) return strip_launch(a.param, g, st);
     return a.kind == 0 ? decode_launch(a.dc, g, sc.ws, sc.ws_bytes, sc.cnt, sc.cnt_len, st) :
-                         prefill_launch(a.param, g, st);
+                         prefill_launch(a.param, a.slices, g, sc, st);
 }
 
 // Heuristic choice (the counterpart of Estimate, gemm_s4_f16.cu:184-206).  Many tokens: the
@@ -129,7 +132,7 @@ int algo_pick(int N, int T, int K)
     auto find_prefill = [&](int tile_t, int tile_n) {
         for (int id = 0; id < algo_count(); ++id) {
             const Algo& a = algo_at(id);
-            if (a.kind == 1 && a.tile_t == tile_t && a.tile_n == tile_n && algo_feasible(id, N, T, K)) return id;
+            if (a.kind == 1 && a.slices == 1 && a.tile_t == tile_t && a.tile_n == tile_n && algo_feasible(id, N, T, K)) return id;
         }
         return -1;
     };

@@ -58,6 +58,21 @@ __device__ __forceinline__ void gload32(uint32_t& dst, uint32_t voff, const void
 {
     asm volatile("global_load_dword %0, %1, %2 offset:%3" : "+v"(dst) : "v"(voff), "s"(sbase), "n"(OFF));
 }
+// Global memory straight into LDS: lane l's 16 bytes land at lds_base + 16 l.  The LDS base travels
+// in M0; written here (rather than through the builtin) so that the address is a scalar base
+// plus a 32-bit lane offset instead of a 64-bit lane address, which costs a register pair and an
+// add per request.
+__device__ __forceinline__ uint32_t lds_addr(const void* p)
+{
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)(p);
+}
+__device__ __forceinline__ void gload_lds128(uint32_t lds_base, uint32_t voff, const void* sbase)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(sbase), "s"(lds_base)
+                 : "memory", "m0");
+}
 // wait until at most N of this wave's loads are in flight; tied to `v` so that no use of it can
 // be scheduled above the wait
 template<int N, typename V>
@@ -81,6 +96,13 @@ __device__ __forceinline__ void wait_lgkm0(half8_t& a, half8_t& b, half8_t& c, h
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
 }
 
+__device__ __forceinline__ uint64_t pack2(float a, float b)
+{
+    return (uint64_t)__builtin_bit_cast(uint32_t, a) | ((uint64_t)__builtin_bit_cast(uint32_t, b) << 32);
+}
+__device__ __forceinline__ float lo_float(uint64_t v) { return __builtin_bit_cast(float, (uint32_t)v); }
+__device__ __forceinline__ float hi_float(uint64_t v) { return __builtin_bit_cast(float, (uint32_t)(v >> 32)); }
+
 // Register budget: one wave per SIMD (512 registers) for the 128-register accumulator tiles,
 // two waves otherwise.  Stating it keeps the allocator from squeezing the kernel into fewer
 // VGPRs and parking values in AGPRs, which is fatal here: a register parked while an
@@ -91,7 +113,8 @@ template<int TTILES, int NTW, int WAVES, int EPI>
 __global__ void __launch_bounds__(64 * WAVES)
     __attribute__((amdgpu_waves_per_eu(TTILES * NTW >= 32 ? 1 : 2, TTILES * NTW >= 32 ? 1 : 2)))
 prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const uint16_t* __restrict__ X,
-               const uint32_t* __restrict__ Q, const uint16_t* R_, int N, int T, int K, int tiles_t, int tiles_n)
+               const uint32_t* __restrict__ Q, const uint16_t* R_, int N, int T, int K, int tiles_t, int tiles_n,
+               float* ws, int* cnt)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [2][TT][kRowBytes]
     constexpr int TT = 16 * TTILES;
@@ -125,6 +148,12 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         tile_t = id % tiles_t;
         tile_n = id / tiles_t;
     }
+    // split K: blockIdx.y takes the quantisation groups [gbeg, gend), dealt in pairs so that only
+    // the last split can have an odd number of them
+    const int splits = gridDim.y;
+    const int pairs  = (G + 1) / 2;
+    const int gbeg   = min(G, 2 * (int)((int64_t)pairs * blockIdx.y / splits));
+    const int gend   = min(G, 2 * (int)((int64_t)pairs * (blockIdx.y + 1) / splits));
     const int T0     = tile_t * TT;
     const int nt0    = (tile_n * TN) / kTileN + wave * NTW;  // first weight tile of this wave
 
@@ -172,11 +201,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     auto issue_x = [&](uint8_t* xo, int g) {
         const char* xbase = reinterpret_cast<const char*>(X) + (int64_t)g * 256;
 #pragma unroll
-        for (int i = 0; i < XB; ++i) {
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(xbase + x_off[i]),
-                (__attribute__((address_space(3))) void*)(xo + (wave * XB + i) * 1024), 16, 0, 0);
-        }
+        for (int i = 0; i < XB; ++i) gload_lds128(lds_addr(xo) + (wave * XB + i) * 1024, x_off[i], xbase);
     };
     // the same requests one at a time (m = 0 .. 2 NTW + TTILES - 1), to be dealt out between MFMAs
     constexpr int kVmOps = 2 * NTW + XB;
@@ -191,9 +216,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         }
         else {
             constexpr int i = m - 2 * NTW;
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(xbase + x_off[i]),
-                (__attribute__((address_space(3))) void*)(xo + (wave * XB + i) * 1024), 16, 0, 0);
+            gload_lds128(lds_addr(xo) + (wave * XB + i) * 1024, x_off[i], xbase);
         }
     };
     auto wait_all = [&](u32x4_t (&w)[NTW], uint32_t (&qv)[NTW]) {
@@ -263,10 +286,21 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     using I1 = std::integral_constant<int, 1>;
 
     // ---- prologue: groups 0 and 1 in flight, first operands of group 0 prepared ----
-    issue_w(wa, qa, 0);
-    issue_x(x0, 0);
-    issue_w(wb, qb, min(1, G - 1));
-    issue_x(x1, min(1, G - 1));
+    // The K loop works through the groups in pairs (the two halves of its body differ in which
+    // registers and which LDS buffer hold the current group).  An odd number of groups is made
+    // even by a phantom group in front: its activation tile is zero-filled LDS instead of a load
+    // and its weights are those of the first real group, so it adds exactly zero.
+    const bool odd    = (gend - gbeg) & 1;
+    const int  gstart = gbeg - (odd ? 1 : 0);
+    issue_w(wa, qa, gbeg);
+    if (odd) {
+        for (int i = tid; i < TT * 16; i += 64 * WAVES) reinterpret_cast<u32x4_t*>(x0)[i] = u32x4_t{0, 0, 0, 0};
+    }
+    else {
+        issue_x(x0, gbeg);
+    }
+    issue_w(wb, qb, gstart + 1);
+    issue_x(x1, gstart + 1);
     wait_all(wa, qa);
     wait_all(wb, qb);
     __syncthreads();
@@ -290,7 +324,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
 #pragma unroll
             for (int tt = 0; tt < TTILES; tt += 4)
                 wait_lgkm0(xf[j & 1][tt], xf[j & 1][tt + 1], xf[j & 1][tt + 2], xf[j & 1][tt + 3]);
-            const int   g2 = min(g + 2, G - 1);  // (the last steps re-read the last group: no branch)
+            const int   g2 = min(g + 2, gend - 1);  // (the last steps re-read the last group: no branch)
             const char* wbase = reinterpret_cast<const char*>(A) + (int64_t)g2 * NT * 1024;
             const char* qbase = reinterpret_cast<const char*>(Q) + (int64_t)g2 * N * 4;
             const char* xbase = reinterpret_cast<const char*>(X) + (int64_t)g2 * 256;
@@ -329,50 +363,125 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         });
     };
 
-    int g = 0;
-    for (; g + 1 < G; g += 2) {  // no branch inside: the 4*TTILES*NTW accumulators stay in place
+    // Whole pairs only (see `odd` above): no K step outside the loop, so the compiler never has a
+    // reason to move an accumulator while the loop's MFMAs may still be writing it.
+    for (int g = gstart; g + 1 < gend; g += 2) {  // no branch inside: the 4*TTILES*NTW accumulators stay in place
         step(I0{}, wa, qa, wb, qb, x0, x1, g);
         step(I1{}, wb, qb, wa, qa, x1, x0, g + 1);
     }
-    if (g < G) step(I0{}, wa, qa, wb, qb, x0, x1, g);
     wait_all(wa, qa);  // no load may still be writing LDS or registers when the wave ends
     wait_all(wb, qb);
+    // The last k32 step requested activation fragments for a step that does not exist.  Nothing
+    // reads them, so the compiler may hand their registers out again at once while the LDS reads
+    // are still on their way and would land on the new owner: wait for them first.  (Tying the
+    // registers to the wait would keep both fragment sets alive and cost registers in the loop;
+    // the build's assembly check verifies instead that nothing touches them before this wait.)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     // the MFMAs are inline assembly, so the compiler does not know that the accumulators are
-    // still being written: cover the longest MFMA-result-to-VALU-read distance by hand
+    // still being written: cover the longest MFMA-result-to-VALU-read distance by hand (the
+    // build's assembly check verifies that no accumulator is read before this)
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // the epilogue of one 16 x 16 tile: lane (c, b) holds token T0 + 16 tt + c, features n .. n+3
+    auto emit = [&](int tt, int nt, const float4_t v) {
+        const int token = T0 + tt * 16 + c;
+        if (token >= T) return;
+        const int    n  = (nt0 + nt) * kTileN + 4 * b;
+        const half_t h0 = (half_t)v[0], h1 = (half_t)v[1], h2 = (half_t)v[2], h3 = (half_t)v[3];
+        if constexpr (EPI == kEpiGemm) {
+            uint2 o;
+            o.x = as_u32(half2_t{h0, h1});
+            o.y = as_u32(half2_t{h2, h3});
+            *reinterpret_cast<uint2*>(C + (int64_t)token * N + n) = o;
+        }
+        else if constexpr (EPI == kEpiSilu) {
+            const float  g0 = (float)h0, u0 = (float)h1, g1 = (float)h2, u1 = (float)h3;
+            const half_t o0 = (half_t)(g0 / (1.f + __expf(-g0)) * u0);
+            const half_t o1 = (half_t)(g1 / (1.f + __expf(-g1)) * u1);
+            *reinterpret_cast<uint32_t*>(C + (int64_t)token * (N / 2) + (n >> 1)) = as_u32(half2_t{o0, o1});
+        }
+        else {
+            const uint2   rr = *reinterpret_cast<const uint2*>(R_ + (int64_t)token * N + n);
+            const half2_t r0 = as_half2(rr.x), r1 = as_half2(rr.y);
+            uint2         o;
+            o.x = as_u32(half2_t{(half_t)((float)r0[0] + (float)h0), (half_t)((float)r0[1] + (float)h1)});
+            o.y = as_u32(half2_t{(half_t)((float)r1[0] + (float)h2), (half_t)((float)r1[1] + (float)h3)});
+            *reinterpret_cast<uint2*>(C + (int64_t)token * N + n) = o;
+        }
+    };
+
+    // ---- split K: exchange partial tiles through the workspace ----
+    // Each wave writes its accumulators as it holds them (per tile two 512-byte rows, lane l the
+    // floats 2l, 2l+1), with agent-scope atomic stores and loads: the L2 caches of the XCDs are not
+    // coherent with each other, and these go through to memory without a full cache write-back.
+    // A store is complete when the wave's store counter drains, so draining it before the arrival
+    // counter is incremented orders the two.  The last workgroup to arrive adds the partial tiles
+    // in split order, its own included, so the sum does not depend on which one is last.
+    if (splits > 1) {
+        constexpr int kTiles = TTILES * NTW;
+        const int64_t per_split = (int64_t)total * WAVES * kTiles * 256;  // floats
+        // (the lane index is hidden from the optimiser here so that none of these addresses is
+        // computed before the K loop and carried through it in registers)
+        int lane_now = lane;
+        asm volatile("" : "+v"(lane_now));
+        float* const  mine_base = ws + ((int64_t)id * WAVES + wave) * kTiles * 256 + lane_now * 2;
+        {
+            float* wp = mine_base + blockIdx.y * per_split;
+#pragma unroll
+            for (int tt = 0; tt < TTILES; ++tt)
+#pragma unroll
+                for (int nt = 0; nt < NTW; ++nt) {
+                    const float4_t v = acc[tt][nt];
+                    uint64_t*      o = reinterpret_cast<uint64_t*>(wp + (tt * NTW + nt) * 256);
+                    __hip_atomic_store(o, pack2(v[0], v[1]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(o + 64, pack2(v[2], v[3]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+        }
+        __builtin_amdgcn_s_waitcnt(0);  // all of this wave's stores are complete
+        __syncthreads();                // ... and every wave is done with the activation tiles in LDS
+        int* const last_flag = reinterpret_cast<int*>(xs);
+        if (tid == 0) {
+            int* const cp   = cnt + id;
+            const int  old  = __hip_atomic_fetch_add(cp, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const bool last = old == splits - 1;
+            if (last) __hip_atomic_store(cp, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+            *last_flag = last;
+        }
+        __syncthreads();
+        if (!*last_flag) return;
+#pragma unroll
+        for (int tt = 0; tt < TTILES; ++tt)
+#pragma unroll
+            for (int nt = 0; nt < NTW; ++nt) {
+                float4_t sum = {0.f, 0.f, 0.f, 0.f};
+                // four splits' loads in flight at a time
+                for (int s0 = 0; s0 < splits; s0 += 4) {
+                    uint64_t v[4][2];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const uint64_t* ip = reinterpret_cast<const uint64_t*>(
+                            mine_base + min(s0 + u, splits - 1) * per_split + (tt * NTW + nt) * 256);
+                        v[u][0] = __hip_atomic_load(ip, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        v[u][1] = __hip_atomic_load(ip + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        if (s0 + u < splits) {
+                            sum[0] += lo_float(v[u][0]); sum[1] += hi_float(v[u][0]);
+                            sum[2] += lo_float(v[u][1]); sum[3] += hi_float(v[u][1]);
+                        }
+                    }
+                }
+                emit(tt, nt, sum);
+            }
+        return;
+    }
 
     // ---- epilogue: lane (c, b) of tile (tt, nt) holds token T0 + 16 tt + c, features n .. n+3 ----
 #pragma unroll
-    for (int tt = 0; tt < TTILES; ++tt) {
-        const int token = T0 + tt * 16 + c;
-        if (token >= T) continue;
+    for (int tt = 0; tt < TTILES; ++tt)
 #pragma unroll
-        for (int nt = 0; nt < NTW; ++nt) {
-            const int      n = (nt0 + nt) * kTileN + 4 * b;
-            const float4_t v = acc[tt][nt];
-            const half_t   h0 = (half_t)v[0], h1 = (half_t)v[1], h2 = (half_t)v[2], h3 = (half_t)v[3];
-            if constexpr (EPI == kEpiGemm) {
-                uint2 o;
-                o.x = as_u32(half2_t{h0, h1});
-                o.y = as_u32(half2_t{h2, h3});
-                *reinterpret_cast<uint2*>(C + (int64_t)token * N + n) = o;
-            }
-            else if constexpr (EPI == kEpiSilu) {
-                const float  g0 = (float)h0, u0 = (float)h1, g1 = (float)h2, u1 = (float)h3;
-                const half_t o0 = (half_t)(g0 / (1.f + __expf(-g0)) * u0);
-                const half_t o1 = (half_t)(g1 / (1.f + __expf(-g1)) * u1);
-                *reinterpret_cast<uint32_t*>(C + (int64_t)token * (N / 2) + (n >> 1)) = as_u32(half2_t{o0, o1});
-            }
-            else {
-                const uint2   rr = *reinterpret_cast<const uint2*>(R_ + (int64_t)token * N + n);
-                const half2_t r0 = as_half2(rr.x), r1 = as_half2(rr.y);
-                uint2         o;
-                o.x = as_u32(half2_t{(half_t)((float)r0[0] + (float)h0), (half_t)((float)r0[1] + (float)h1)});
-                o.y = as_u32(half2_t{(half_t)((float)r1[0] + (float)h2), (half_t)((float)r1[1] + (float)h3)});
-                *reinterpret_cast<uint2*>(C + (int64_t)token * N + n) = o;
-            }
-        }
-    }
+        for (int nt = 0; nt < NTW; ++nt) emit(tt, nt, acc[tt][nt]);
 }
 
 struct Variant {
@@ -385,13 +494,13 @@ constexpr Variant kVariants[] = {{8, 2, 8}, {16, 2, 4}, {8, 2, 4}, {4, 2, 4}, {4
 constexpr int     kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 template<int TTILES, int NTW, int WAVES>
-hipError_t launch_v(const GemmArgs& a, hipStream_t st)
+hipError_t launch_v(int splits, const GemmArgs& a, const Scratch& sc, hipStream_t st)
 {
     constexpr int TT = 16 * TTILES, TN = 16 * NTW * WAVES;
     const int     tiles_t = (a.T + TT - 1) / TT;
     const int     tiles_n = a.N / TN;
     const size_t  lds     = (size_t)2 * TT * kRowBytes;
-    const dim3    grid(tiles_t * tiles_n), block(64 * WAVES);
+    const dim3    grid(tiles_t * tiles_n, splits), block(64 * WAVES);
     const u32x4_t* A4 = reinterpret_cast<const u32x4_t*>(a.A);
 #define W4A16_LAUNCH(EPI)                                                                                              \
     do {                                                                                                               \
@@ -399,7 +508,8 @@ hipError_t launch_v(const GemmArgs& a, hipStream_t st)
         hipError_t e   = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),                                       \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
         if (e != hipSuccess) return e;                                                                                 \
-        hipLaunchKernelGGL(kfn, grid, block, lds, st, a.C, A4, a.X, a.Q, a.R, a.N, a.T, a.K, tiles_t, tiles_n);        \
+        hipLaunchKernelGGL(kfn, grid, block, lds, st, a.C, A4, a.X, a.Q, a.R, a.N, a.T, a.K, tiles_t, tiles_n,        \
+                           sc.ws, sc.cnt);                                                                             \
     } while (0)
     switch (a.epilogue) {
         case kEpiGemm: W4A16_LAUNCH(kEpiGemm); break;
@@ -423,33 +533,39 @@ void prefill_tile(int v, int& tile_n, int& tile_t)
     tile_t = 16 * kVariants[v].ttiles;
 }
 
-bool prefill_feasible(int v, int N, int T, int K)
+bool prefill_feasible(int v, int splits, int N, int T, int K)
 {
-    if (v < 0 || v >= kNumVariants || N <= 0 || T <= 0 || K <= 0) return false;
+    if (v < 0 || v >= kNumVariants || N <= 0 || T <= 0 || K <= 0 || splits < 1) return false;
     const int tn = 16 * kVariants[v].ntw * kVariants[v].waves, tt = 16 * kVariants[v].ttiles;
     if (N % tn != 0 || K % kGroup != 0) return false;
     // per-thread offsets into X and into one group of A are 32-bit
     if ((int64_t)T * K * 2 >= (1ll << 32) || (int64_t)N * 64 >= (1ll << 32)) return false;
     const int64_t grid = (int64_t)(N / tn) * ((T + tt - 1) / tt);
-    return grid < (1ll << 31);
+    if (splits > 1) {
+        // at least two groups per split; partial tiles and counters must fit the handle's scratch
+        if (K / kGroup < 2 * splits || splits > 65535) return false;
+        if (grid * splits * tn * tt * 4 > (int64_t)kWorkspaceBytes || grid > kCounters) return false;
+    }
+    return grid * splits < (1ll << 31);
 }
 
-int prefill_grid(int v, int N, int T, int K)
+int prefill_grid(int v, int splits, int N, int T, int K)
 {
     (void)K;
     const int tn = 16 * kVariants[v].ntw * kVariants[v].waves, tt = 16 * kVariants[v].ttiles;
-    return (N / tn) * ((T + tt - 1) / tt);
+    return (N / tn) * ((T + tt - 1) / tt) * splits;
 }
 
-hipError_t prefill_launch(int v, const GemmArgs& a, hipStream_t st)
+hipError_t prefill_launch(int v, int splits, const GemmArgs& a, const Scratch& sc, hipStream_t st)
 {
+    if (splits > 1 && (sc.ws == nullptr || sc.cnt == nullptr)) return hipErrorInvalidValue;
     switch (v) {
-        case 0: return launch_v<8, 2, 8>(a, st);
-        case 1: return launch_v<16, 2, 4>(a, st);
-        case 2: return launch_v<8, 2, 4>(a, st);
-        case 3: return launch_v<4, 2, 4>(a, st);
-        case 4: return launch_v<4, 1, 4>(a, st);
-        default: return launch_v<8, 4, 4>(a, st);
+        case 0: return launch_v<8, 2, 8>(splits, a, sc, st);
+        case 1: return launch_v<16, 2, 4>(splits, a, sc, st);
+        case 2: return launch_v<8, 2, 4>(splits, a, sc, st);
+        case 3: return launch_v<4, 2, 4>(splits, a, sc, st);
+        case 4: return launch_v<4, 1, 4>(splits, a, sc, st);
+        default: return launch_v<8, 4, 4>(splits, a, sc, st);
     }
 }
 

@@ -30,12 +30,15 @@ struct Algo {
     int          kind;     // 0 decode (column blocks), 1 prefill, 2 decode (strips)
     int          tile_n;   // output features per workgroup
     int          tile_t;   // tokens per workgroup
-    int          slices;   // K slices per workgroup
+    int          slices;   // decode: K slices per workgroup; prefill: K splits across workgroups
     int          param;    // prefill: variant index; strips: strips per CU aimed for
     DecodeConfig dc;       // decode only
 };
 
-// Scratch owned by a handle: split-K partial tiles and arrival counters.
+// Scratch owned by a handle: split-K partial tiles and arrival counters.  Every handle has exactly
+// this much, so feasibility of a split-K launch does not depend on the handle.
+constexpr size_t kWorkspaceBytes = 64u << 20;
+constexpr int    kCounters       = 1 << 16;
 struct Scratch {
     float* ws;
     size_t ws_bytes;
@@ -79,8 +82,10 @@ hipError_t strip_launch(int per_cu, const GemmArgs& a, hipStream_t st);
 // MFMA prefill kernels
 int        prefill_variants();
 void       prefill_tile(int variant, int& tile_n, int& tile_t);
-bool       prefill_feasible(int variant, int N, int T, int K);
-int        prefill_grid(int variant, int N, int T, int K);
-hipError_t prefill_launch(int variant, const GemmArgs& a, hipStream_t st);
+// `splits` > 1 divides the quantisation groups among that many workgroups per output tile; the
+// last one to arrive adds the partial tiles (in split order) and runs the epilogue.
+bool       prefill_feasible(int variant, int splits, int N, int T, int K);
+int        prefill_grid(int variant, int splits, int N, int T, int K);
+hipError_t prefill_launch(int variant, int splits, const GemmArgs& a, const Scratch& sc, hipStream_t st);
 
 }  // namespace w4a16

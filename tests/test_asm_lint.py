@@ -46,3 +46,16 @@ def test_join_takes_the_younger_position():
 def test_other_functions_are_ignored():
     asm = "_ZN5w4a166helperEv:\n" + load(0) + "\tv_mov_b32_e32 v20, v1\n" + TAIL
     assert lint(asm) == []
+
+
+def test_parking_an_in_flight_register_in_an_agpr_is_reported():
+    # the register allocator saves a VGPR to an AGPR to reuse it, while a load into it is pending:
+    # the saved value is stale and the load later lands on the register's new owner
+    asm = HEAD + load(48) + "\tv_accvgpr_write_b32 a106, v51\n\ts_waitcnt vmcnt(0)\n" + TAIL
+    msgs = lint(asm)
+    assert len(msgs) == 1 and "v51" in msgs[0]
+
+
+def test_parking_a_settled_register_is_accepted():
+    asm = HEAD + load(48) + "\ts_waitcnt vmcnt(0)\n\tv_accvgpr_write_b32 a106, v51\n" + TAIL
+    assert lint(asm) == []

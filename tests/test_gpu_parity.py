@@ -162,6 +162,29 @@ def test_every_kernel_small_shape(tm, gemm, T):
     assert ran >= 20
 
 
+@pytest.mark.parametrize("K", [128, 640, 1408])
+def test_every_kernel_odd_number_of_groups(tm, gemm, K):
+    # K / 128 odd: the prefill kernels, which walk K two groups at a time, must pad with a group
+    # that adds nothing; with K split across workgroups some splits are odd and some even
+    N = 256
+    for T in (40, 130):
+        d = O.make_inputs(700 + K + T, T, K, N, residual=True)
+        A, Q = convert(tm, d, N, K)
+        want = {k: O.gemm_s4_f16(d["X"], d["qweight"], d["qzeros"], d["scales"], 128, k, d.get("R")) for k in (0, 1, 2)}
+        ran = 0
+        for algo in _algos(gemm):
+            for kind in (0, 1, 2):
+                try:
+                    got = run(tm, gemm, d, A, Q, T, K, N, kind, algo)
+                except tm.W4A16Error as e:
+                    assert e.code == -2, e
+                    continue
+                ran += 1
+                err = O.max_abs_rel(got, want[kind])
+                assert np.isfinite(got).all() and err <= TOL, (algo, kind, T, err)
+        assert ran >= 20
+
+
 def test_identity_activations_return_weights(tm, gemm):
     # X = I  =>  Y == W.  The prefill kernels use the reference's exact fp16 weight, so they are
     # bit exact; the decode kernels scale after the group sum: (q - z) * s rounded once from fp32,
