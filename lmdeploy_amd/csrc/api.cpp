@@ -123,44 +123,28 @@ hipError_t algo_launch(int id, const GemmArgs& g, const Scratch& sc, hipStream_t
                          prefill_launch(a.param, a.slices, g, sc, st);
 }
 
-// Heuristic choice (the counterpart of Estimate, gemm_s4_f16.cu:184-206).  Many tokens: the
-// MFMA prefill kernel whose tile count wastes the least of the last round of workgroups.
-// Few tokens: the decode kernel, see below.
+// Heuristic choice (the counterpart of Estimate, gemm_s4_f16.cu:184-206).  Above 16 tokens:
+// every MFMA prefill tile, unsplit and with K split 2, 4 or 8 ways, is priced with a model of
+// measured step times, and so is the decode kernel (which re-reads the weights once per 16
+// tokens); the cheapest wins.  Up to 16 tokens: the decode kernel, see below.
 int algo_pick(int N, int T, int K)
 {
     if (T <= 0 || N <= 0 || K <= 0) return -1;
-    auto find_prefill = [&](int tile_t, int tile_n) {
+    if (T > 16) {
+        int    best = -1;
+        double best_us = 0;
         for (int id = 0; id < algo_count(); ++id) {
             const Algo& a = algo_at(id);
-            if (a.kind == 1 && a.slices == 1 && a.tile_t == tile_t && a.tile_n == tile_n && algo_feasible(id, N, T, K)) return id;
+            if (a.kind != 1 || !algo_feasible(id, N, T, K)) continue;
+            const double us = prefill_estimate_us(a.param, a.slices, N, T, K);
+            if (best < 0 || us < best_us) best = id, best_us = us;
         }
-        return -1;
-    };
-    if (T > 32) {
-        // Prefill tiles by a cost model fitted to sweeps on MI355X: a CU works through its
-        // workgroups at a fixed rate per output element, so time ~ (workgroups / 256) x tile
-        // area x a penalty for small tiles (more dequantisation and LDS traffic per MFMA).  One
-        // tile's trip through K is the floor however idle the chip is, which is why short prompts
-        // want small tiles; ties go to the wider tile (less activation traffic).  If even the best
-        // tiling leaves more than a third of the CUs empty at <= 128 tokens (narrow matrices such as o_proj
-        // and down_proj) the decode kernels are faster.
-        struct Tile { int t, n; double penalty; };
-        const Tile tiles[5] = {{128, 256, 1.0}, {128, 128, 1.0}, {256, 128, 1.07}, {64, 128, 1.2}, {64, 64, 1.6}};
-        int    best = -1;
-        double best_cost = 0;
-        int64_t best_wgs = 0;
-        for (const Tile& t : tiles) {
-            if (N % t.n != 0) continue;
-            const int id = find_prefill(t.t, t.n);
-            if (id < 0) continue;
-            const int64_t wgs  = (int64_t)(N / t.n) * ((T + t.t - 1) / t.t);
-            // tiles with one workgroup per CU go in whole rounds; smaller ones share CUs, which evens out
-            const bool    one_per_cu = t.t * t.n > 128 * 128;  // (also the eight-wave 128 x 256 tile: it fills a CU)
-            const double  rounds     = one_per_cu ? (double)((wgs + 255) / 256) : std::max(1.0, wgs / 256.0);
-            const double  cost       = rounds * t.t * t.n * t.penalty;
-            if (best < 0 || cost < best_cost * 0.999) best = id, best_cost = cost, best_wgs = wgs;
-        }
-        if (best >= 0 && (T > 128 || best_wgs >= 160) && (T >= 64 || best_wgs >= 256)) return best;
+        // decode: launch + the weight stream once per block of 16 tokens; later blocks find part of it
+        // in the caches (exponent fitted to 2 .. 8 blocks on Llama-7B shapes)
+        // (narrow matrices use the column-block kernel with K split across workgroups: 1.4 x)
+        const double blocks    = (T + 15) / 16;
+        const double decode_us = 3.0 + std::pow(blocks, 0.85) * ((double)K * N / 2) / 4.2e6 * (N / 16 < 512 ? 1.4 : 1.0);
+        if (best >= 0 && best_us < decode_us) return best;
     }
     // Decode.  Strips of column tiles over the whole of K, one per CU, were the fastest on every
     // Llama-7B/70B shape measured at 1..16 tokens; two narrower strips per CU are slightly ahead on

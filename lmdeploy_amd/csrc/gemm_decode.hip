@@ -434,7 +434,9 @@ Plan make_plan(const DecodeConfig& cf, int N, int T, int K, size_t ws_bytes, int
     const long wgs = (long)pl.nb * pl.z;
     int        sk  = 1;
     if (cf.fill > 0) {
-        const long want = ((long)cf.fill * 256 + wgs - 1) / wgs;
+        // as many splits as keep the grid within 256 * fill workgroups: one more would start a
+        // second, mostly empty round
+        const long want = std::max(1l, (long)cf.fill * 256 / wgs);
         sk              = (int)std::max(1l, std::min<long>(want, std::max(1, G / cf.sk)));
         // partial tiles must fit the workspace, counters the counter array
         while (sk > 1 && ((size_t)pl.z * sk * NT * 1024 > ws_bytes || wgs > cnt_len)) --sk;

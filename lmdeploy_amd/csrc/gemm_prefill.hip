@@ -22,6 +22,7 @@
 #include "w4a16_common.h"
 #include "w4a16_internal.h"
 
+#include <cmath>
 #include <type_traits>
 
 namespace w4a16 {
@@ -109,18 +110,22 @@ __device__ __forceinline__ float hi_float(uint64_t v) { return __builtin_bit_cas
 // inline-assembly load into it is still in flight is handed to another value, and the load then
 // lands on that value (the build rejects kernels that use AGPRs beyond their accumulators).
 // WAVES = waves per workgroup (4 or 8), side by side along the features.
-template<int TTILES, int NTW, int WAVES, int EPI>
+// D = groups in flight per wave (2 or 4): the loads of group g + D are issued while group g is
+// being multiplied.  Two cover the memory latency when a K step is long (large tiles); small tiles
+// finish a step in a fraction of that and need four.
+template<int TTILES, int NTW, int WAVES, int D, int EPI>
 __global__ void __launch_bounds__(64 * WAVES)
     __attribute__((amdgpu_waves_per_eu(TTILES * NTW >= 32 ? 1 : 2, TTILES * NTW >= 32 ? 1 : 2)))
 prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const uint16_t* __restrict__ X,
                const uint32_t* __restrict__ Q, const uint16_t* R_, int N, int T, int K, int tiles_t, int tiles_n,
                float* ws, int* cnt)
 {
-    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [2][TT][kRowBytes]
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [D][TT][kRowBytes]
     constexpr int TT = 16 * TTILES;
     constexpr int TN = 16 * NTW * WAVES;
     constexpr int XB = 4 * TTILES / WAVES;  // 1 KiB activation blocks (4 token rows) that each wave fetches per group
     static_assert(4 * TTILES % WAVES == 0, "the activation tile must divide evenly among the waves");
+    static_assert(D == 2 || D == 4, "stages alternate in parity, so their number is even");
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
@@ -183,18 +188,20 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) acc[tt][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    u32x4_t  wa[NTW], wb[NTW];  // weights of the current / next group (roles alternate)
-    uint32_t qa[NTW], qb[NTW];
+    u32x4_t  w[D][NTW];  // weights and (scale, zero) words of the D groups in flight; stage = group index mod D
+    uint32_t q[D][NTW];
 #pragma unroll
-    for (int nt = 0; nt < NTW; ++nt) {
-        wa[nt] = wb[nt] = u32x4_t{0, 0, 0, 0};
-        qa[nt] = qb[nt] = 0;
-    }
+    for (int d = 0; d < D; ++d)
+#pragma unroll
+        for (int nt = 0; nt < NTW; ++nt) {
+            w[d][nt] = u32x4_t{0, 0, 0, 0};
+            q[d][nt] = 0;
+        }
 
-    auto issue_w = [&](u32x4_t (&w)[NTW], uint32_t (&qv)[NTW], int g) {
+    auto issue_w = [&](u32x4_t (&ws_)[NTW], uint32_t (&qv)[NTW], int g) {
         const char* wbase = reinterpret_cast<const char*>(A) + (int64_t)g * NT * 1024;
         const char* qbase = reinterpret_cast<const char*>(Q) + (int64_t)g * N * 4;
-        static_for<0, NTW>([&](auto nt) { gload128<nt * 1024>(w[nt], w_off, wbase); });
+        static_for<0, NTW>([&](auto nt) { gload128<nt * 1024>(ws_[nt], w_off, wbase); });
         static_for<0, NTW>([&](auto nt) { gload32<nt * 64>(qv[nt], q_off, qbase); });
     };
     // the activation tile of group g, straight into the LDS buffer `xo` (no registers, no ds_write)
@@ -205,11 +212,11 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     };
     // the same requests one at a time (m = 0 .. 2 NTW + TTILES - 1), to be dealt out between MFMAs
     constexpr int kVmOps = 2 * NTW + XB;
-    auto vm_op = [&](auto M, u32x4_t (&w)[NTW], uint32_t (&qv)[NTW], uint8_t* xo, const char* wbase, const char* qbase,
+    auto vm_op = [&](auto M, u32x4_t (&ws_)[NTW], uint32_t (&qv)[NTW], uint8_t* xo, const char* wbase, const char* qbase,
                      const char* xbase) {
         constexpr int m = decltype(M)::value;
         if constexpr (m < NTW) {
-            gload128<m * 1024>(w[m], w_off, wbase);
+            gload128<m * 1024>(ws_[m], w_off, wbase);
         }
         else if constexpr (m < 2 * NTW) {
             gload32<(m - NTW) * 64>(qv[m - NTW], q_off, qbase);
@@ -219,16 +226,18 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
             gload_lds128(lds_addr(xo) + (wave * XB + i) * 1024, x_off[i], xbase);
         }
     };
-    auto wait_all = [&](u32x4_t (&w)[NTW], uint32_t (&qv)[NTW]) {
+    // wait until at most `Pending` younger stages' loads are in flight, then release the stage's registers
+    auto wait_stage = [&](auto Pending, u32x4_t (&ws_)[NTW], uint32_t (&qv)[NTW]) {
+        constexpr int n = decltype(Pending)::value * kVmOps;
+        static_assert(n <= 63, "vmcnt is a 6-bit counter");
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) {
-            wait_vm<0>(w[nt]);
-            wait_vm<0>(qv[nt]);
+            wait_vm<n>(ws_[nt]);
+            wait_vm<n>(qv[nt]);
         }
     };
-
-    uint8_t* const x0 = xs;
-    uint8_t* const x1 = xs + TT * kRowBytes;
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
 
     // State carried from one k32 step to the next (and across K steps): dequantised weights and
     // activation fragments of the current / next k32 step, zero points and scale of the current /
@@ -250,13 +259,13 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     // (op = NTW * k + nt) so that they can be dealt out between the MFMAs of a k32 step:
     // k = 0: w >> 8;  1..4: (w & mask) | magic;  5..8: - (offset + zero);  9..12: * scale.
     uint32_t dq[NTW][5];
-    auto dequant_op = [&](auto P, auto J, auto OP, u32x4_t (&w)[NTW]) {
+    auto dequant_op = [&](auto P, auto J, auto OP, u32x4_t (&ws_)[NTW]) {
         constexpr int p = decltype(P)::value, j = decltype(J)::value;
         constexpr int nt = decltype(OP)::value % NTW, k = decltype(OP)::value / NTW;
-        if constexpr (k == 0) dq[nt][4] = w[nt][j] >> 8;
+        if constexpr (k == 0) dq[nt][4] = ws_[nt][j] >> 8;
         else if constexpr (k <= 4) {
             constexpr int i  = k - 1;
-            const uint32_t src = i < 2 ? w[nt][j] : dq[nt][4];
+            const uint32_t src = i < 2 ? ws_[nt][j] : dq[nt][4];
             dq[nt][i] = (src & (i & 1 ? uc.mask_hi : uc.mask_lo)) | (i & 1 ? uc.magic_hi : uc.magic_lo);
         }
         else if constexpr (k <= 8) {
@@ -270,8 +279,8 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
             wf[j & 1][nt][2 * i + 1] = r[1];
         }
     };
-    auto dequant = [&](auto P, auto J, u32x4_t (&w)[NTW]) {
-        static_for<0, 13 * NTW>([&](auto op) { dequant_op(P, J, op, w); });
+    auto dequant = [&](auto P, auto J, u32x4_t (&ws_)[NTW]) {
+        static_for<0, 13 * NTW>([&](auto op) { dequant_op(P, J, op, ws_); });
     };
     auto read_x = [&](auto J_, const uint8_t* xb) {
         constexpr int  J    = decltype(J_)::value;
@@ -282,60 +291,63 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         constexpr int J = decltype(J_)::value, tt = decltype(TT_)::value;
         lds_read128<tt * 16 * kRowBytes>(xf[J & 1][tt], base + xr_off[J]);
     };
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
-
-    // ---- prologue: groups 0 and 1 in flight, first operands of group 0 prepared ----
-    // The K loop works through the groups in pairs (the two halves of its body differ in which
-    // registers and which LDS buffer hold the current group).  An odd number of groups is made
-    // even by a phantom group in front: its activation tile is zero-filled LDS instead of a load
-    // and its weights are those of the first real group, so it adds exactly zero.
-    const bool odd    = (gend - gbeg) & 1;
-    const int  gstart = gbeg - (odd ? 1 : 0);
-    issue_w(wa, qa, gbeg);
-    if (odd) {
-        for (int i = tid; i < TT * 16; i += 64 * WAVES) reinterpret_cast<u32x4_t*>(x0)[i] = u32x4_t{0, 0, 0, 0};
-    }
-    else {
-        issue_x(x0, gbeg);
-    }
-    issue_w(wb, qb, gstart + 1);
-    issue_x(x1, gstart + 1);
-    wait_all(wa, qa);
-    wait_all(wb, qb);
+    // ---- prologue: the first D groups in flight, first operands of the first one prepared ----
+    // The K loop works through the groups D at a time (the D parts of its body differ in which
+    // registers and which LDS buffer hold the current group).  A group count that is not a
+    // multiple of D is padded with phantom groups in front: their activation tile is zero-filled
+    // LDS instead of a load and their weights are those of the first real group, so they add
+    // exactly zero.
+    const int pad    = (D - (gend - gbeg) % D) % D;
+    const int gstart = gbeg - pad;
+    static_for<0, D>([&](auto dc) {
+        constexpr int d  = decltype(dc)::value;
+        uint8_t* const xd = xs + d * TT * kRowBytes;
+        issue_w(w[d], q[d], max(gstart + d, gbeg));
+        if (gstart + d < gbeg) {
+            for (int i = tid; i < TT * 16; i += 64 * WAVES) reinterpret_cast<u32x4_t*>(xd)[i] = u32x4_t{0, 0, 0, 0};
+        }
+        else {
+            issue_x(xd, gstart + d);
+        }
+    });
+    static_for<0, D>([&](auto dc) { wait_stage(I0{}, w[decltype(dc)::value], q[decltype(dc)::value]); });
     __syncthreads();
-    read_x(I0{}, x0);
-    split(I0{}, qa);
-    dequant(I0{}, I0{}, wa);
+    read_x(I0{}, xs);
+    split(I0{}, q[0]);
+    dequant(I0{}, I0{}, w[0]);
 
-    // One K step (a quantisation group, four k32 steps) on the weights `w` (group parity P) and the
-    // LDS buffer `xb`.  Every k32 step runs its MFMAs interleaved with the dequantisation of the
+    // One K step (a quantisation group, four k32 steps) on stage S: weights w[S], LDS buffer S, group
+    // parity S & 1.  Every k32 step runs its MFMAs interleaved with the dequantisation of the
     // NEXT k32 step's weights and the requests for its activation fragments.  In the last k32 step
-    // the next group's weights (`wn`, requested one K step ago) and activation tile (`xo`) are
-    // complete: the workgroup synchronises, starts on them, and re-uses `w` and `xb`, which no wave
-    // reads any more, for the loads of group g + 2.
-    auto step = [&](auto P, u32x4_t (&w)[NTW], uint32_t (&qv)[NTW], u32x4_t (&wn)[NTW], uint32_t (&qn)[NTW],
-                    uint8_t* xb, const uint8_t* xo, int g) {
-        constexpr int p  = decltype(P)::value;
+    // the next group's weights (stage S + 1, requested D - 1 K steps ago) and activation tile are
+    // complete: the workgroup synchronises, starts on them, and re-uses stage S, which no wave
+    // reads any more, for the loads of group g + D.
+    auto step = [&](auto S_, int g) {
+        constexpr int S = decltype(S_)::value, SN = (S + 1) % D;
+        constexpr int p = S & 1;
+        using P          = std::integral_constant<int, p>;
         using PN         = std::integral_constant<int, p ^ 1>;
+        uint8_t* const       xb = xs + S * TT * kRowBytes;
+        const uint8_t* const xo = xs + SN * TT * kRowBytes;
         static_for<0, 4>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             using JN        = std::integral_constant<int, (j + 1) & 3>;
 #pragma unroll
             for (int tt = 0; tt < TTILES; tt += 4)
                 wait_lgkm0(xf[j & 1][tt], xf[j & 1][tt + 1], xf[j & 1][tt + 2], xf[j & 1][tt + 3]);
-            const int   g2 = min(g + 2, gend - 1);  // (the last steps re-read the last group: no branch)
+            const int   g2 = min(g + D, gend - 1);  // (the last steps re-read the last group: no branch)
             const char* wbase = reinterpret_cast<const char*>(A) + (int64_t)g2 * NT * 1024;
             const char* qbase = reinterpret_cast<const char*>(Q) + (int64_t)g2 * N * 4;
             const char* xbase = reinterpret_cast<const char*>(X) + (int64_t)g2 * 256;
             if constexpr (j == 3) {
-                wait_all(wn, qn);
+                // stages S + 2 .. S + D - 1 may still be in flight behind stage S + 1
+                wait_stage(std::integral_constant<int, D - 2>{}, w[SN], q[SN]);
                 __syncthreads();
             }
             const uint32_t rbase =
                 (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)(j < 3 ? (const uint8_t*)xb : xo);
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (j == 3) split(PN{}, qn);
+            if constexpr (j == 3) split(PN{}, q[SN]);
             // one MFMA, then its share of the next k32 step's dequantisation, and so on
             constexpr int kOps = 13 * NTW, kSlots = TTILES * NTW;
             static_for<0, kSlots>([&](auto ic) {
@@ -345,32 +357,31 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
                              : "v"(wf[j & 1][nt]), "v"(xf[j & 1][tt]));
                 __builtin_amdgcn_sched_barrier(0);
                 static_for<i * kOps / kSlots, (i + 1) * kOps / kSlots>([&](auto op) {
-                    if constexpr (j < 3) dequant_op(P, JN{}, op, w);
-                    else dequant_op(PN{}, I0{}, op, wn);
+                    if constexpr (j < 3) dequant_op(P{}, JN{}, op, w[S]);
+                    else dequant_op(PN{}, I0{}, op, w[SN]);
                 });
                 // the next k32 step's activation fragments, requested during the first three quarters
-                // of this one; in the last k32 step also the loads of group g + 2
+                // of this one; in the last k32 step also the loads of group g + D
                 constexpr int kR = kSlots * 3 / 4 > 0 ? kSlots * 3 / 4 : 1;
                 if constexpr (i < kR) {
                     static_for<i * TTILES / kR, (i + 1) * TTILES / kR>([&](auto tt) { read_x1(JN{}, tt, rbase); });
                 }
                 if constexpr (j == 3) {
                     static_for<i * kVmOps / kSlots, (i + 1) * kVmOps / kSlots>(
-                        [&](auto m) { vm_op(m, w, qv, xb, wbase, qbase, xbase); });
+                        [&](auto m) { vm_op(m, w[S], q[S], xb, wbase, qbase, xbase); });
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
         });
     };
 
-    // Whole pairs only (see `odd` above): no K step outside the loop, so the compiler never has a
-    // reason to move an accumulator while the loop's MFMAs may still be writing it.
-    for (int g = gstart; g + 1 < gend; g += 2) {  // no branch inside: the 4*TTILES*NTW accumulators stay in place
-        step(I0{}, wa, qa, wb, qb, x0, x1, g);
-        step(I1{}, wb, qb, wa, qa, x1, x0, g + 1);
+    // Whole multiples of D only (see `pad` above): no K step outside the loop, so the compiler never
+    // has a reason to move an accumulator while the loop's MFMAs may still be writing it.
+    for (int g = gstart; g + D - 1 < gend; g += D) {  // no branch inside: the 4*TTILES*NTW accumulators stay in place
+        static_for<0, D>([&](auto dc) { step(dc, g + decltype(dc)::value); });
     }
-    wait_all(wa, qa);  // no load may still be writing LDS or registers when the wave ends
-    wait_all(wb, qb);
+    // no load may still be writing LDS or registers when the wave ends
+    static_for<0, D>([&](auto dc) { wait_stage(I0{}, w[decltype(dc)::value], q[decltype(dc)::value]); });
     // The last k32 step requested activation fragments for a step that does not exist.  Nothing
     // reads them, so the compiler may hand their registers out again at once while the LDS reads
     // are still on their way and would land on the new owner: wait for them first.  (Tying the
@@ -485,26 +496,37 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
 }
 
 struct Variant {
-    int ttiles, ntw, waves;
+    int ttiles, ntw, waves, depth;
+    // Measured on MI355X (K = 2048 against 6144, cold weights): microseconds per K step for the whole
+    // grid at 1, 2, 3, 4 and 8 workgroups per CU.  Tiles that fill a CU by themselves go in rounds.
+    bool  one_per_cu;
+    float step_us[5];
 };
 // (a 256 x 256 tile does not fit the register file without spilling, and spill stores would
 // break the counted waits: stores and loads complete out of order with each other)
-// (first match wins in the dispatcher: the 8-wave 128 x 256 tile comes before the 4-wave one)
-constexpr Variant kVariants[] = {{8, 2, 8}, {16, 2, 4}, {8, 2, 4}, {4, 2, 4}, {4, 1, 4}, {8, 4, 4}};
-constexpr int     kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+constexpr Variant kVariants[] = {
+    {8, 2, 8, 2, true, {1.905f, 3.821f, 5.517f, 7.090f, 13.658f}},   // 128 x 256, eight waves
+    {16, 2, 4, 2, true, {2.071f, 4.498f, 6.126f, 8.397f, 15.010f}},  // 256 x 128
+    {8, 2, 4, 2, false, {1.016f, 1.860f, 3.067f, 4.002f, 7.185f}},   // 128 x 128
+    {4, 2, 4, 4, false, {0.672f, 1.111f, 1.664f, 2.271f, 4.773f}},   //  64 x 128
+    {4, 1, 4, 4, false, {0.443f, 0.701f, 1.041f, 1.396f, 2.951f}},   //  64 x 64
+    {4, 1, 8, 4, true, {0.576f, 1.259f, 1.985f, 2.718f, 5.574f}},    //  64 x 128, eight waves
+    {4, 2, 8, 4, true, {1.034f, 2.290f, 3.605f, 4.644f, 8.583f}},    //  64 x 256, eight waves
+};
+constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
-template<int TTILES, int NTW, int WAVES>
+template<int TTILES, int NTW, int WAVES, int D>
 hipError_t launch_v(int splits, const GemmArgs& a, const Scratch& sc, hipStream_t st)
 {
     constexpr int TT = 16 * TTILES, TN = 16 * NTW * WAVES;
     const int     tiles_t = (a.T + TT - 1) / TT;
     const int     tiles_n = a.N / TN;
-    const size_t  lds     = (size_t)2 * TT * kRowBytes;
+    const size_t  lds     = (size_t)D * TT * kRowBytes;
     const dim3    grid(tiles_t * tiles_n, splits), block(64 * WAVES);
     const u32x4_t* A4 = reinterpret_cast<const u32x4_t*>(a.A);
 #define W4A16_LAUNCH(EPI)                                                                                              \
     do {                                                                                                               \
-        auto       kfn = prefill_kernel<TTILES, NTW, WAVES, EPI>;                                                             \
+        auto       kfn = prefill_kernel<TTILES, NTW, WAVES, D, EPI>;                                                           \
         hipError_t e   = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),                                       \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
         if (e != hipSuccess) return e;                                                                                 \
@@ -560,13 +582,51 @@ hipError_t prefill_launch(int v, int splits, const GemmArgs& a, const Scratch& s
 {
     if (splits > 1 && (sc.ws == nullptr || sc.cnt == nullptr)) return hipErrorInvalidValue;
     switch (v) {
-        case 0: return launch_v<8, 2, 8>(splits, a, sc, st);
-        case 1: return launch_v<16, 2, 4>(splits, a, sc, st);
-        case 2: return launch_v<8, 2, 4>(splits, a, sc, st);
-        case 3: return launch_v<4, 2, 4>(splits, a, sc, st);
-        case 4: return launch_v<4, 1, 4>(splits, a, sc, st);
-        default: return launch_v<8, 4, 4>(splits, a, sc, st);
+        case 0: return launch_v<8, 2, 8, 2>(splits, a, sc, st);
+        case 1: return launch_v<16, 2, 4, 2>(splits, a, sc, st);
+        case 2: return launch_v<8, 2, 4, 2>(splits, a, sc, st);
+        case 3: return launch_v<4, 2, 4, 4>(splits, a, sc, st);
+        case 4: return launch_v<4, 1, 4, 4>(splits, a, sc, st);
+        case 5: return launch_v<4, 1, 8, 4>(splits, a, sc, st);
+        default: return launch_v<4, 2, 8, 4>(splits, a, sc, st);
     }
+}
+
+// Predicted run time in microseconds, from the measured step times: launch and epilogue, the K
+// steps of one workgroup at the load the grid puts on the chip, and for split K the exchange of
+// partial tiles.
+double prefill_estimate_us(int v, int splits, int N, int T, int K)
+{
+    const Variant& var = kVariants[v];
+    const int      tn = 16 * var.ntw * var.waves, tt = 16 * var.ttiles;
+    const double   wgs  = (double)(N / tn) * ((T + tt - 1) / tt) * splits;
+    const double   load = wgs / 256.0;
+    // tiles that fill a CU by themselves go in whole rounds
+    const double le = var.one_per_cu ? std::ceil(load) : load;
+    double       step;
+    if (le <= 4.0) {
+        step = var.step_us[le <= 1.0 ? 0 : le <= 2.0 ? 1 : le <= 3.0 ? 2 : 3];
+    }
+    else if (le <= 8.0) {
+        step = var.step_us[3] + (var.step_us[4] - var.step_us[3]) * (le - 4.0) / 4.0;
+    }
+    else {
+        step = var.step_us[4] * le / 8.0;
+    }
+    // corrections from real Llama shapes: a partly idle chip clocks higher and shares less memory
+    // bandwidth; 64-token tiles under heavy load ran slower than on the calibration grid
+    if (var.one_per_cu && load < 1.0) step *= 0.7 + 0.3 * load;
+    if (!var.one_per_cu && var.ttiles == 4 && load > 2.0) step *= 1.25;
+    const int groups = K / kGroup;
+    int       steps  = (groups + splits - 1) / splits;
+    steps            = (steps + var.depth - 1) / var.depth * var.depth;  // phantom groups
+    double us = 3.0 + steps * step;
+    if (splits > 1) {
+        const double tokens = (double)((T + tt - 1) / tt) * tt;
+        // drain of the partial stores, arrival counter, then the last workgroup reads every split's tile
+        us += 2.0 + 0.6 * splits + splits * tokens * N * 8.0 / 4.0e6;
+    }
+    return us;
 }
 
 }  // namespace w4a16

@@ -87,5 +87,6 @@ void       prefill_tile(int variant, int& tile_n, int& tile_t);
 bool       prefill_feasible(int variant, int splits, int N, int T, int K);
 int        prefill_grid(int variant, int splits, int N, int T, int K);
 hipError_t prefill_launch(int variant, int splits, const GemmArgs& a, const Scratch& sc, hipStream_t st);
+double     prefill_estimate_us(int variant, int splits, int N, int T, int K);  // model fitted to measurements
 
 }  // namespace w4a16
