@@ -67,6 +67,8 @@ std::vector<Algo> build_table()
     }
     // strips of column tiles over the whole of K, 1 or 2 per CU
     for (int per_cu : {1, 2}) t.push_back(Algo{2, 0, 16, 8, per_cu, DecodeConfig{}});
+    // the same with 32 tokens per workgroup (17 tokens and more): half the passes over the weights
+    for (int per_cu : {1, 2}) t.push_back(Algo{2, 0, 32, 8, per_cu, DecodeConfig{}});
     for (int v = 0; v < prefill_variants(); ++v) {
         int tn = 0, tt = 0;
         prefill_tile(v, tn, tt);
@@ -104,21 +106,21 @@ const Algo& algo_at(int id)
 bool algo_feasible(int id, int N, int T, int K)
 {
     const Algo& a = algo_at(id);
-    if (a.kind == 2) return strip_feasible(a.param, N, T, K);
+    if (a.kind == 2) return strip_feasible(a.param, a.tile_t, N, T, K);
     return a.kind == 0 ? decode_feasible(a.dc, N, T, K) : prefill_feasible(a.param, a.slices, N, T, K);
 }
 
 int algo_grid(int id, int N, int T, int K, const Scratch& sc)
 {
     const Algo& a = algo_at(id);
-    if (a.kind == 2) return strip_grid(a.param, N, T, K);
+    if (a.kind == 2) return strip_grid(a.param, a.tile_t, N, T, K);
     return a.kind == 0 ? decode_grid(a.dc, N, T, K, sc.ws_bytes, sc.cnt_len) : prefill_grid(a.param, a.slices, N, T, K);
 }
 
 hipError_t algo_launch(int id, const GemmArgs& g, const Scratch& sc, hipStream_t st)
 {
     const Algo& a = algo_at(id);
-    if (a.kind == 2) return strip_launch(a.param, g, st);
+    if (a.kind == 2) return strip_launch(a.param, a.tile_t, g, st);
     return a.kind == 0 ? decode_launch(a.dc, g, sc.ws, sc.ws_bytes, sc.cnt, sc.cnt_len, st) :
                          prefill_launch(a.param, a.slices, g, sc, st);
 }
@@ -144,7 +146,19 @@ int algo_pick(int N, int T, int K)
         // (narrow matrices use the column-block kernel with K split across workgroups: 1.4 x)
         const double blocks    = (T + 15) / 16;
         const double decode_us = 3.0 + std::pow(blocks, 0.85) * ((double)K * N / 2) / 4.2e6 * (N / 16 < 512 ? 1.4 : 1.0);
-        if (best >= 0 && best_us < decode_us) return best;
+        // 17..32 tokens: the strip kernel with 32 tokens per workgroup streams the weights once, at
+        // 1.25 x (17 tokens) to 1.6 x (32 tokens) the cost of a 16-token pass
+        int    strip32 = -1;
+        double strip32_us = 0;
+        if (T <= 32) {
+            for (int id = 0; id < algo_count() && strip32 < 0; ++id) {
+                const Algo& a = algo_at(id);
+                if (a.kind == 2 && a.tile_t == 32 && a.param == 1 && algo_feasible(id, N, T, K)) strip32 = id;
+            }
+            strip32_us = 3.0 + (1.25 + 0.35 * (T - 16) / 16.0) * ((double)K * N / 2) / 4.2e6;
+        }
+        if (best >= 0 && best_us < decode_us && (strip32 < 0 || best_us < strip32_us)) return best;
+        if (strip32 >= 0 && strip32_us < decode_us) return strip32;
     }
     // Decode.  Strips of column tiles over the whole of K, one per CU, were the fastest on every
     // Llama-7B/70B shape measured at 1..16 tokens; two narrower strips per CU are slightly ahead on
@@ -158,7 +172,7 @@ int algo_pick(int N, int T, int K)
         for (int per_cu : {want, 1}) {
             for (int id = 0; id < algo_count(); ++id) {
                 const Algo& a = algo_at(id);
-                if (a.kind == 2 && a.param == per_cu && algo_feasible(id, N, T, K)) return id;
+                if (a.kind == 2 && a.tile_t == 16 && a.param == per_cu && algo_feasible(id, N, T, K)) return id;
             }
         }
     }
@@ -331,7 +345,7 @@ int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const 
         w4a16_metric m{};
         m.id       = id;
         m.kind     = a.kind;
-        m.tile_n   = a.kind == 2 ? 16 * strip_width(a.param, n_out, tokens, k) : a.tile_n;
+        m.tile_n   = a.kind == 2 ? 16 * strip_width(a.param, a.tile_t, n_out, tokens, k) : a.tile_n;
         m.tile_t   = a.tile_t;
         m.slices   = a.slices;
         m.best     = id == best;

@@ -30,6 +30,7 @@ namespace {
 
 constexpr int kWaves   = 8;  // = K slices per workgroup
 constexpr int kMaxR    = 8;  // column tiles per strip
+constexpr int kMaxR32  = 4;  // ... with 32 tokens per workgroup (register budget)
 constexpr int kNumCU   = 256;
 
 struct StripParams {
@@ -110,8 +111,10 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     const int N = p.N, T = p.T, K = p.K;
     const int G  = K / kGroup;
     const int NT = N / kTileN;
-    const int t0 = blockIdx.y * 16;
-    const int Tl = min(16, T - t0);
+    // H row blocks of 16 tokens share every unpacked weight (H = 2 for the 32-token variant)
+    constexpr int H  = TP > 16 ? TP / 16 : 1;
+    const int     t0 = blockIdx.y * (16 * H);
+    const int     Tl = min(16 * H, T - t0);
 
     // this wave's groups: wave, wave + 8, wave + 16, ...  Interleaved rather than blocked, so that
     // at any moment the whole chip reads one contiguous run of a few dozen group rows of the
@@ -135,17 +138,19 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     for (int i = 0; i < NX; ++i)
         x_off[i] = (uint32_t)min(t0 + 4 * i + (lane >> 4), T - 1) * (uint32_t)(K * 2) + (uint32_t)((lane & 15) * 16);
     u32x4_t* const xw = smem + wave * (TP * 16);  // this wave's patch: [TP rows][16 chunks]
-    int            xw_at[NX], xr_at[4];
+    int            xw_at[NX], xr_at[H][4];
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
         const int r = 4 * i + (lane >> 4);
         xw_at[i]    = r * 16 + ((lane & 15) ^ (r & 15));
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int r = c & (TP - 1);  // MFMA rows >= TP repeat a lower row: they only feed outputs that are never stored
-        xr_at[j]    = r * 16 + ((4 * j + b) ^ (r & 15));
-    }
+    for (int h = 0; h < H; ++h)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int r = 16 * h + (c & (TP - 1));  // MFMA rows >= TP repeat a lower row: they only feed outputs that are never stored
+            xr_at[h][j] = r * 16 + ((4 * j + b) ^ (r & 15));
+        }
 
     const char* Ab = reinterpret_cast<const char*>(p.A) + (int64_t)col0 * 1024;
     const char* Qb = reinterpret_cast<const char*>(p.Q) + (int64_t)col0 * 64;
@@ -166,23 +171,27 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     constexpr int kLoads = 2 * R + NX;  // loads per stage
 
     const UnpackConsts uc;
-    float4_t           acc[R];
+    float4_t           acc[H][R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int h = 0; h < H; ++h)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[h][r] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     // One tile of one group.  U tiles are worked on at a time with their MFMA chains interleaved:
     // a chain is eight dependent MFMAs, and a dependent MFMA cannot issue before its predecessor
     // has left the pipe.
     auto compute = [&](Stage<R, NX>& s) {
-        half8_t xf[4];
+        half8_t xf[H][4];
 #pragma unroll
         for (int i = 0; i < NX; ++i) xw[xw_at[i]] = s.x[i];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) xf[j] = __builtin_bit_cast(half8_t, xw[xr_at[j]]);  // same wave: LDS keeps the order
+        for (int h = 0; h < H; ++h)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xf[h][j] = __builtin_bit_cast(half8_t, xw[xr_at[h][j]]);  // same wave: LDS keeps the order
         constexpr int U = 2;
 #pragma unroll
         for (int r0 = 0; r0 < R; r0 += U) {
-            float4_t g4[U];
+            float4_t g4[H][U];
             float    sf[U];
             half8_t  bz[U];
 #pragma unroll
@@ -190,23 +199,26 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
                 const int r = r0 + u < R ? r0 + u : R - 1;
                 // B operand that removes the unpack offsets and the zero point: -(1024 + z) under
                 // the low-nibble pairs, -(64 + z) under the high-nibble pairs
-                const half2_t  h   = as_half2(s.q[r]);
-                const half2_t  n64 = half2_t{h[0], h[0]} * half2_t{(half_t)-1.f, (half_t)-1.f};
+                const half2_t  h2  = as_half2(s.q[r]);
+                const half2_t  n64 = half2_t{h2[0], h2[0]} * half2_t{(half_t)-1.f, (half_t)-1.f};
                 const uint32_t zb  = ((s.q[r] >> 4) & 0xfu) * 0x10001u + 0xE400E400u;  // -(1024 + z) twice
                 bz[u][0] = as_half2(zb)[0]; bz[u][1] = as_half2(zb)[1]; bz[u][2] = n64[0]; bz[u][3] = n64[1];
                 bz[u][4] = bz[u][0]; bz[u][5] = bz[u][1]; bz[u][6] = bz[u][2]; bz[u][7] = bz[u][3];
                 // Convert the scale now and hide it from the optimiser: otherwise the conversion is
                 // folded into the final multiply-add, the Q word stays live past the refill of this
                 // stage, and the refill lands in a copy that is moved back while still in flight.
-                sf[u] = (float)h[1];
+                sf[u] = (float)h2[1];
                 asm volatile("" : "+v"(sf[u]));
-                g4[u] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int h = 0; h < H; ++h) g4[h][u] = float4_t{0.f, 0.f, 0.f, 0.f};
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
 #pragma unroll
                 for (int u = 0; u < U; ++u)
-                    if (r0 + u < R) g4[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[j], bz[u], g4[u], 0, 0, 0);
+#pragma unroll
+                    for (int h = 0; h < H; ++h)
+                        if (r0 + u < R) g4[h][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[h][j], bz[u], g4[h][u], 0, 0, 0);
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -218,13 +230,17 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
                         half8_t wf;
                         wf[0] = as_half2(v[0])[0]; wf[1] = as_half2(v[0])[1]; wf[2] = as_half2(v[1])[0]; wf[3] = as_half2(v[1])[1];
                         wf[4] = as_half2(v[2])[0]; wf[5] = as_half2(v[2])[1]; wf[6] = as_half2(v[3])[0]; wf[7] = as_half2(v[3])[1];
-                        g4[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[j], wf, g4[u], 0, 0, 0);
+#pragma unroll
+                        for (int h = 0; h < H; ++h)
+                            g4[h][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[h][j], wf, g4[h][u], 0, 0, 0);
                     }
                 }
             }
 #pragma unroll
             for (int u = 0; u < U; ++u)
-                if (r0 + u < R) acc[r0 + u] += sf[u] * g4[u];
+#pragma unroll
+                for (int h = 0; h < H; ++h)
+                    if (r0 + u < R) acc[h][r0 + u] += sf[u] * g4[h][u];
         }
     };
     // Wait until the stage's loads are complete (loads return in order: at most `kLoads` younger
@@ -274,40 +290,44 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the masked refills of the last trip
 
     // ---- add the eight slices in LDS, in slice order ----
-    // red[slice][r][lane] as float4, over the activation patches: every wave must be done with its own
+    // red[slice][r][h][lane] as float4, over the activation patches: every wave must be done with its own
     __syncthreads();
     float4_t* red4 = reinterpret_cast<float4_t*>(smem);
 #pragma unroll
-    for (int r = 0; r < R; ++r) red4[(wave * R + r) * 64 + lane] = acc[r];
-    __syncthreads();
-    for (int r = wave; r < R; r += kWaves) {  // tile r of the strip is finished by wave r (mod 8)
-        float4_t v = {0.f, 0.f, 0.f, 0.f};
+    for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int s = 0; s < kWaves; ++s) v += red4[(s * R + r) * 64 + lane];
+        for (int h = 0; h < H; ++h) red4[((wave * R + r) * H + h) * 64 + lane] = acc[h][r];
+    __syncthreads();
+    for (int rh = wave; rh < R * H; rh += kWaves) {  // (tile r, row block h) is finished by wave r * H + h (mod 8)
+        const int r = rh / H, h = rh % H;
+        float4_t  v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < kWaves; ++s) v += red4[((s * R + r) * H + h) * 64 + lane];
 
-        // ---- epilogue: lane (c, b) holds column n = 16 * (col0 + r) + c, tokens t0 + 4b + i ----
+        // ---- epilogue: lane (c, b) holds column n = 16 * (col0 + r) + c, tokens t0 + 16h + 4b + i ----
         const int n = (col0 + r) * kTileN + c;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const half_t h     = (half_t)v[i];
-            const int    token = t0 + 4 * b + i;
+            const half_t hv    = (half_t)v[i];
+            const int    row   = 16 * h + 4 * b + i;
+            const int    token = t0 + row;
             if constexpr (EPI == kEpiSilu) {
                 // gate = even column, up = odd column: fetch the neighbour lane's value
-                const float mine  = (float)h;
+                const float mine  = (float)hv;
                 const float other = __shfl_xor(mine, 1);
-                if (4 * b + i < Tl && (c & 1) == 0) {
+                if (row < Tl && (c & 1) == 0) {
                     const half_t o = (half_t)(mine / (1.f + __expf(-mine)) * other);
                     p.C[(int64_t)token * (N / 2) + (n >> 1)] = __builtin_bit_cast(uint16_t, o);
                 }
             }
-            else if (4 * b + i < Tl) {
+            else if (row < Tl) {
                 const int64_t at = (int64_t)token * N + n;
                 if constexpr (EPI == kEpiGemm) {
-                    p.C[at] = __builtin_bit_cast(uint16_t, h);
+                    p.C[at] = __builtin_bit_cast(uint16_t, hv);
                 }
                 else {
                     const half_t rr = __builtin_bit_cast(half_t, p.Rsd[at]);
-                    const half_t o  = (half_t)((float)rr + (float)h);
+                    const half_t o  = (half_t)((float)rr + (float)hv);
                     p.C[at]         = __builtin_bit_cast(uint16_t, o);
                 }
             }
@@ -350,7 +370,11 @@ hipError_t launch_r(int tp, const StripParams& p, dim3 grid, size_t lds, int epi
     switch (tp) {
         case 4: return launch_rt<RMAX, 4>(p, grid, lds, epilogue, st);
         case 8: return launch_rt<RMAX, 8>(p, grid, lds, epilogue, st);
-        default: return launch_rt<RMAX, 16>(p, grid, lds, epilogue, st);
+        case 16: return launch_rt<RMAX, 16>(p, grid, lds, epilogue, st);
+        default:
+            // 32 tokens per block: twice the accumulators and activation registers, strips of at most kMaxR32 tiles
+            if constexpr (RMAX <= kMaxR32) return launch_rt<RMAX, 32>(p, grid, lds, epilogue, st);
+            return hipErrorInvalidValue;
     }
 }
 
@@ -359,51 +383,57 @@ struct StripPlan {
     bool ok;
 };
 
-// `per_cu` strips per CU are aimed for; more if a strip would otherwise be wider than kMaxR.
-StripPlan make_plan(int per_cu, int N, int T, int K)
+// `per_cu` strips per CU are aimed for; more if a strip would otherwise be wider than the limit.
+// block_t = tokens per workgroup: 16 (activation rows padded down to 4 or 8 for fewer tokens) or 32.
+StripPlan make_plan(int per_cu, int block_t, int N, int T, int K)
 {
     StripPlan pl{};
     if (N <= 0 || K <= 0 || T <= 0 || N % kTileN != 0 || K % kGroup != 0 || per_cu < 1) return pl;
-    const int NT = N / kTileN;
-    int       m  = per_cu;
-    while ((NT + kNumCU * m - 1) / (kNumCU * m) > kMaxR) ++m;
+    if (block_t != 16 && block_t != 32) return pl;
+    if (block_t == 32 && T <= 16) return pl;  // the 16-token kernel covers these
+    const int NT   = N / kTileN;
+    const int maxr = block_t == 32 ? kMaxR32 : kMaxR;
+    int       m    = per_cu;
+    while ((NT + kNumCU * m - 1) / (kNumCU * m) > maxr) ++m;
     pl.strips = std::min(NT, kNumCU * m);
     pl.base   = NT / pl.strips;
     pl.rem    = NT % pl.strips;
     pl.rmax   = pl.base + (pl.rem ? 1 : 0);
     // 32-bit per-lane offsets into X; grid limits
-    pl.ok = (int64_t)T * K * 2 < (1ll << 32) && (T + 15) / 16 <= 65535 && (per_cu == 1 || pl.strips == kNumCU * per_cu);
+    pl.ok = (int64_t)T * K * 2 < (1ll << 32) && (T + block_t - 1) / block_t <= 65535 &&
+            (per_cu == 1 || pl.strips == kNumCU * per_cu);
     return pl;
 }
 
 }  // namespace
 
-bool strip_feasible(int per_cu, int N, int T, int K)
+bool strip_feasible(int per_cu, int block_t, int N, int T, int K)
 {
-    return make_plan(per_cu, N, T, K).ok;
+    return make_plan(per_cu, block_t, N, T, K).ok;
 }
 
-int strip_grid(int per_cu, int N, int T, int K)
+int strip_grid(int per_cu, int block_t, int N, int T, int K)
 {
-    const StripPlan pl = make_plan(per_cu, N, T, K);
-    return pl.strips * ((T + 15) / 16);
+    const StripPlan pl = make_plan(per_cu, block_t, N, T, K);
+    return pl.strips * ((T + block_t - 1) / block_t);
 }
 
-int strip_width(int per_cu, int N, int T, int K)
+int strip_width(int per_cu, int block_t, int N, int T, int K)
 {
-    return make_plan(per_cu, N, T, K).rmax;
+    return make_plan(per_cu, block_t, N, T, K).rmax;
 }
 
-hipError_t strip_launch(int per_cu, const GemmArgs& a, hipStream_t st)
+hipError_t strip_launch(int per_cu, int block_t, const GemmArgs& a, hipStream_t st)
 {
-    const StripPlan pl = make_plan(per_cu, a.N, a.T, a.K);
+    const StripPlan pl = make_plan(per_cu, block_t, a.N, a.T, a.K);
     if (!pl.ok) return hipErrorInvalidValue;
     const int   G  = a.K / kGroup;
-    const int   tp = a.T <= 4 ? 4 : (a.T <= 8 ? 8 : 16);
+    const int   tp = block_t == 32 ? 32 : (a.T <= 4 ? 4 : (a.T <= 8 ? 8 : 16));
+    const int   h  = tp > 16 ? tp / 16 : 1;
     StripParams p{a.C, reinterpret_cast<const u32x4_t*>(a.A), a.X, a.Q, a.R, a.N, a.T, a.K, pl.base, pl.rem,
                   (G + kWaves - 1) / kWaves};
-    const dim3   grid(pl.strips, (a.T + 15) / 16);
-    const size_t lds = (size_t)kWaves * std::max(pl.rmax * 1024, tp * 256);
+    const dim3   grid(pl.strips, (a.T + block_t - 1) / block_t);
+    const size_t lds = (size_t)kWaves * std::max(pl.rmax * h * 1024, tp * 256);
     switch (pl.rmax) {
         case 1: return launch_r<1>(tp, p, grid, lds, a.epilogue, st);
         case 2: return launch_r<2>(tp, p, grid, lds, a.epilogue, st);

@@ -73,11 +73,11 @@ int        decode_grid(const DecodeConfig& cf, int N, int T, int K, size_t ws_by
 hipError_t decode_launch(const DecodeConfig& cf, const GemmArgs& a, float* ws, size_t ws_bytes, int* cnt, int cnt_len,
                          hipStream_t st);
 
-// decode kernels, strip decomposition (gemm_strip.hip)
-bool       strip_feasible(int per_cu, int N, int T, int K);
-int        strip_grid(int per_cu, int N, int T, int K);
-int        strip_width(int per_cu, int N, int T, int K);  // column tiles of the widest strip
-hipError_t strip_launch(int per_cu, const GemmArgs& a, hipStream_t st);
+// decode kernels, strip decomposition (gemm_strip.hip); block_t = tokens per workgroup, 16 or 32
+bool       strip_feasible(int per_cu, int block_t, int N, int T, int K);
+int        strip_grid(int per_cu, int block_t, int N, int T, int K);
+int        strip_width(int per_cu, int block_t, int N, int T, int K);  // column tiles of the widest strip
+hipError_t strip_launch(int per_cu, int block_t, const GemmArgs& a, hipStream_t st);
 
 // MFMA prefill kernels
 int        prefill_variants();

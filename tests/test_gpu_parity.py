@@ -353,11 +353,12 @@ def test_llama7b_32_layer_decode_sequence(tm, gemm):
             assert err <= TOL, (li, K, N, kind, err)
 
 
-@pytest.mark.parametrize("K,N", [(1024, 3072), (512, 4112), (128, 16), (2048, 2064)])
+@pytest.mark.parametrize("K,N", [(1024, 3072), (512, 4112), (128, 16), (2048, 2064), (4224, 1024)])
 def test_default_dispatch_over_token_counts(tm, gemm, K, N):
     """`algo_id = -1` across the hand-over points between the decode, strip and prefill kernels,
-    on shapes with and without the divisibility the wider tiles need (4112 = 16 * 257, 2064 = 16 * 129)."""
-    Ts = (1, 5, 16, 17, 33, 48, 64, 100, 129, 192, 300, 1000)
+    on shapes with and without the divisibility the wider tiles need (4112 = 16 * 257, 2064 = 16 * 129),
+    and on a deep narrow one (33 groups) where the prefill tiles split K across workgroups."""
+    Ts = (1, 5, 16, 17, 24, 32, 33, 48, 64, 100, 129, 192, 300, 1000)
     d = O.make_inputs(900 + K + N, max(Ts), K, N, residual=True)
     A, Q = convert(tm, d, N, K)
     W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], 128)
