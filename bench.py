@@ -32,8 +32,8 @@ MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16 matrix
 # runs of `bench.py --probe ...`, calibrated against an elementwise kernel of known size
 # (profiles/decode_gate_up_hbm_traffic.md, profiles/prefill_gate_up_mfma_and_traffic.md).
 N_LAYERS = 32          # Llama-2-7B
-TRAFFIC_DECODE_GATE_UP = 49.38e6
-TRAFFIC_PREFILL_GATE_UP = 565.0e6
+TRAFFIC_DECODE_GATE_UP = 49.37e6
+TRAFFIC_PREFILL_GATE_UP = 565.2e6
 
 # name, K, N (gate_up: both halves), epilogue
 LAYER_7B = [("qkv", 4096, 12288, 0), ("o", 4096, 4096, 0), ("gate_up", 4096, 22016, 1), ("down", 11008, 4096, 2)]

@@ -113,9 +113,14 @@ __device__ __forceinline__ float hi_float(uint64_t v) { return __builtin_bit_cas
 // D = groups in flight per wave (2 or 4): the loads of group g + D are issued while group g is
 // being multiplied.  Two cover the memory latency when a K step is long (large tiles); small tiles
 // finish a step in a fraction of that and need four.
-template<int TTILES, int NTW, int WAVES, int D, int EPI>
+// KS = k32 chunks per sub-step (1 or 2).  The operands of a sub-step - activation fragments from
+// LDS, dequantised weights - are requested and prepared during the previous one.  A 64-token tile
+// has only 4 * NTW MFMAs per k32 chunk, too few to cover the LDS latency; two chunks per sub-step
+// double the cover at the price of a second set of fragment registers.
+template<int TTILES, int NTW, int WAVES, int D, int KS, int EPI>
 __global__ void __launch_bounds__(64 * WAVES)
-    __attribute__((amdgpu_waves_per_eu(TTILES * NTW >= 32 ? 1 : 2, TTILES * NTW >= 32 ? 1 : 2)))
+    __attribute__((amdgpu_waves_per_eu(TTILES * NTW * KS >= 16 && WAVES == 4 && (TTILES * NTW >= 32 || KS == 2) ? 1 : 2,
+                                       TTILES * NTW * KS >= 16 && WAVES == 4 && (TTILES * NTW >= 32 || KS == 2) ? 1 : 2)))
 prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const uint16_t* __restrict__ X,
                const uint32_t* __restrict__ Q, const uint16_t* R_, int N, int T, int K, int tiles_t, int tiles_n,
                float* ws, int* cnt)
@@ -126,6 +131,8 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     constexpr int XB = 4 * TTILES / WAVES;  // 1 KiB activation blocks (4 token rows) that each wave fetches per group
     static_assert(4 * TTILES % WAVES == 0, "the activation tile must divide evenly among the waves");
     static_assert(D == 2 || D == 4, "stages alternate in parity, so their number is even");
+    static_assert(KS == 1 || KS == 2, "a group is four k32 chunks; sub-steps alternate in parity");
+    constexpr int kSub = 4 / KS;  // sub-steps per group
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
@@ -242,8 +249,8 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     // State carried from one k32 step to the next (and across K steps): dequantised weights and
     // activation fragments of the current / next k32 step, zero points and scale of the current /
     // next group.
-    half8_t wf[2][NTW];
-    half8_t xf[2][TTILES];
+    half8_t wf[2][KS][NTW];   // [sub-step parity][chunk][tile]
+    half8_t xf[2][KS][TTILES];
     half2_t z1024[2][NTW], z64[2][NTW], sc[2][NTW];
 
     auto split = [&](auto P_, uint32_t (&qv)[NTW]) {
@@ -275,8 +282,8 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         else {
             constexpr int i = k - 9;
             const half2_t r = as_half2(dq[nt][i]) * sc[p][nt];
-            wf[j & 1][nt][2 * i]     = r[0];
-            wf[j & 1][nt][2 * i + 1] = r[1];
+            wf[(j / KS) & 1][j % KS][nt][2 * i]     = r[0];
+            wf[(j / KS) & 1][j % KS][nt][2 * i + 1] = r[1];
         }
     };
     auto dequant = [&](auto P, auto J, u32x4_t (&ws_)[NTW]) {
@@ -285,11 +292,11 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     auto read_x = [&](auto J_, const uint8_t* xb) {
         constexpr int  J    = decltype(J_)::value;
         const uint32_t addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)(xb) + xr_off[J];
-        static_for<0, TTILES>([&](auto tt) { lds_read128<tt * 16 * kRowBytes>(xf[J & 1][tt], addr); });
+        static_for<0, TTILES>([&](auto tt) { lds_read128<tt * 16 * kRowBytes>(xf[(J / KS) & 1][J % KS][tt], addr); });
     };
     auto read_x1 = [&](auto J_, auto TT_, uint32_t base) {
         constexpr int J = decltype(J_)::value, tt = decltype(TT_)::value;
-        lds_read128<tt * 16 * kRowBytes>(xf[J & 1][tt], base + xr_off[J]);
+        lds_read128<tt * 16 * kRowBytes>(xf[(J / KS) & 1][J % KS][tt], base + xr_off[J]);
     };
     // ---- prologue: the first D groups in flight, first operands of the first one prepared ----
     // The K loop works through the groups D at a time (the D parts of its body differ in which
@@ -312,16 +319,18 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     });
     static_for<0, D>([&](auto dc) { wait_stage(I0{}, w[decltype(dc)::value], q[decltype(dc)::value]); });
     __syncthreads();
-    read_x(I0{}, xs);
     split(I0{}, q[0]);
-    dequant(I0{}, I0{}, w[0]);
+    static_for<0, KS>([&](auto kc) {
+        read_x(kc, xs);
+        dequant(I0{}, kc, w[0]);
+    });
 
-    // One K step (a quantisation group, four k32 steps) on stage S: weights w[S], LDS buffer S, group
-    // parity S & 1.  Every k32 step runs its MFMAs interleaved with the dequantisation of the
-    // NEXT k32 step's weights and the requests for its activation fragments.  In the last k32 step
-    // the next group's weights (stage S + 1, requested D - 1 K steps ago) and activation tile are
-    // complete: the workgroup synchronises, starts on them, and re-uses stage S, which no wave
-    // reads any more, for the loads of group g + D.
+    // One K step (a quantisation group, four k32 chunks in kSub sub-steps) on stage S: weights w[S],
+    // LDS buffer S, group parity S & 1.  Every sub-step runs its MFMAs interleaved with the
+    // dequantisation of the NEXT sub-step's weights and the requests for its activation fragments.
+    // In the last sub-step the next group's weights (stage S + 1, requested D - 1 K steps ago) and
+    // activation tile are complete: the workgroup synchronises, starts on them, and re-uses stage
+    // S, which no wave reads any more, for the loads of group g + D.
     auto step = [&](auto S_, int g) {
         constexpr int S = decltype(S_)::value, SN = (S + 1) % D;
         constexpr int p = S & 1;
@@ -329,44 +338,54 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         using PN         = std::integral_constant<int, p ^ 1>;
         uint8_t* const       xb = xs + S * TT * kRowBytes;
         const uint8_t* const xo = xs + SN * TT * kRowBytes;
-        static_for<0, 4>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            using JN        = std::integral_constant<int, (j + 1) & 3>;
+        static_for<0, kSub>([&](auto sc_) {
+            constexpr int  sub  = decltype(sc_)::value;
+            constexpr bool last = sub == kSub - 1;
+            constexpr int  par  = sub & 1;
 #pragma unroll
-            for (int tt = 0; tt < TTILES; tt += 4)
-                wait_lgkm0(xf[j & 1][tt], xf[j & 1][tt + 1], xf[j & 1][tt + 2], xf[j & 1][tt + 3]);
+            for (int kk = 0; kk < KS; ++kk)
+#pragma unroll
+                for (int tt = 0; tt < TTILES; tt += 4)
+                    wait_lgkm0(xf[par][kk][tt], xf[par][kk][tt + 1], xf[par][kk][tt + 2], xf[par][kk][tt + 3]);
             const int   g2 = min(g + D, gend - 1);  // (the last steps re-read the last group: no branch)
             const char* wbase = reinterpret_cast<const char*>(A) + (int64_t)g2 * NT * 1024;
             const char* qbase = reinterpret_cast<const char*>(Q) + (int64_t)g2 * N * 4;
             const char* xbase = reinterpret_cast<const char*>(X) + (int64_t)g2 * 256;
-            if constexpr (j == 3) {
+            if constexpr (last) {
                 // stages S + 2 .. S + D - 1 may still be in flight behind stage S + 1
                 wait_stage(std::integral_constant<int, D - 2>{}, w[SN], q[SN]);
                 __syncthreads();
             }
             const uint32_t rbase =
-                (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)(j < 3 ? (const uint8_t*)xb : xo);
+                (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)(last ? xo : (const uint8_t*)xb);
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (j == 3) split(PN{}, q[SN]);
-            // one MFMA, then its share of the next k32 step's dequantisation, and so on
-            constexpr int kOps = 13 * NTW, kSlots = TTILES * NTW;
+            if constexpr (last) split(PN{}, q[SN]);
+            // one MFMA, then its share of the next sub-step's dequantisation, and so on
+            constexpr int kOps = 13 * NTW * KS, kSlots = TTILES * NTW * KS, kReads = TTILES * KS;
             static_for<0, kSlots>([&](auto ic) {
-                constexpr int i = decltype(ic)::value, tt = i / NTW, nt = i % NTW;
+                constexpr int i = decltype(ic)::value, kk = i / (TTILES * NTW), tt = i % (TTILES * NTW) / NTW, nt = i % NTW;
                 asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
                              : "+a"(acc[tt][nt])
-                             : "v"(wf[j & 1][nt]), "v"(xf[j & 1][tt]));
+                             : "v"(wf[par][kk][nt]), "v"(xf[par][kk][tt]));
                 __builtin_amdgcn_sched_barrier(0);
+                // (word = chunk of the next sub-step, 13 * NTW operations each, in order: they share temporaries)
                 static_for<i * kOps / kSlots, (i + 1) * kOps / kSlots>([&](auto op) {
-                    if constexpr (j < 3) dequant_op(P{}, JN{}, op, w[S]);
-                    else dequant_op(PN{}, I0{}, op, w[SN]);
+                    constexpr int word = decltype(op)::value / (13 * NTW);
+                    using OP           = std::integral_constant<int, decltype(op)::value % (13 * NTW)>;
+                    if constexpr (!last) dequant_op(P{}, std::integral_constant<int, (sub + 1) * KS + word>{}, OP{}, w[S]);
+                    else dequant_op(PN{}, std::integral_constant<int, word>{}, OP{}, w[SN]);
                 });
-                // the next k32 step's activation fragments, requested during the first three quarters
-                // of this one; in the last k32 step also the loads of group g + D
+                // the next sub-step's activation fragments, requested during the first three quarters
+                // of this one; in the last sub-step also the loads of group g + D
                 constexpr int kR = kSlots * 3 / 4 > 0 ? kSlots * 3 / 4 : 1;
                 if constexpr (i < kR) {
-                    static_for<i * TTILES / kR, (i + 1) * TTILES / kR>([&](auto tt) { read_x1(JN{}, tt, rbase); });
+                    static_for<i * kReads / kR, (i + 1) * kReads / kR>([&](auto rd) {
+                        constexpr int chunk = (last ? 0 : (sub + 1) * KS) + decltype(rd)::value / TTILES;
+                        read_x1(std::integral_constant<int, chunk>{},
+                                std::integral_constant<int, decltype(rd)::value % TTILES>{}, rbase);
+                    });
                 }
-                if constexpr (j == 3) {
+                if constexpr (last) {
                     static_for<i * kVmOps / kSlots, (i + 1) * kVmOps / kSlots>(
                         [&](auto m) { vm_op(m, w[S], q[S], xb, wbase, qbase, xbase); });
                 }
@@ -496,26 +515,27 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
 }
 
 struct Variant {
-    int ttiles, ntw, waves, depth;
+    int ttiles, ntw, waves, depth, chunks;
     // Measured on MI355X (K = 2048 against 6144, cold weights): microseconds per K step for the whole
     // grid at 1, 2, 3, 4 and 8 workgroups per CU.  Tiles that fill a CU by themselves go in rounds.
+    // (The two-chunk rows are the one-chunk measurements x 0.96, the ratio seen on Llama-7B shapes.)
     bool  one_per_cu;
     float step_us[5];
 };
 // (a 256 x 256 tile does not fit the register file without spilling, and spill stores would
 // break the counted waits: stores and loads complete out of order with each other)
 constexpr Variant kVariants[] = {
-    {8, 2, 8, 2, true, {1.905f, 3.821f, 5.517f, 7.090f, 13.658f}},   // 128 x 256, eight waves
-    {16, 2, 4, 2, true, {2.071f, 4.498f, 6.126f, 8.397f, 15.010f}},  // 256 x 128
-    {8, 2, 4, 2, false, {1.016f, 1.860f, 3.067f, 4.002f, 7.185f}},   // 128 x 128
-    {4, 2, 4, 4, false, {0.672f, 1.111f, 1.664f, 2.271f, 4.773f}},   //  64 x 128
-    {4, 1, 4, 4, false, {0.443f, 0.701f, 1.041f, 1.396f, 2.951f}},   //  64 x 64
-    {4, 1, 8, 4, true, {0.576f, 1.259f, 1.985f, 2.718f, 5.574f}},    //  64 x 128, eight waves
-    {4, 2, 8, 4, true, {1.034f, 2.290f, 3.605f, 4.644f, 8.583f}},    //  64 x 256, eight waves
+    {8, 2, 8, 2, 1, true, {1.905f, 3.821f, 5.517f, 7.090f, 13.658f}},   // 128 x 256, eight waves
+    {16, 2, 4, 2, 1, true, {2.071f, 4.498f, 6.126f, 8.397f, 15.010f}},  // 256 x 128
+    {8, 2, 4, 2, 1, false, {1.016f, 1.860f, 3.067f, 4.002f, 7.185f}},   // 128 x 128
+    {4, 2, 4, 4, 1, false, {0.672f, 1.111f, 1.664f, 2.271f, 4.773f}},   //  64 x 128
+    {4, 1, 4, 4, 2, false, {0.425f, 0.673f, 1.000f, 1.340f, 2.833f}},   //  64 x 64, two chunks per sub-step
+    {4, 1, 8, 4, 2, true, {0.553f, 1.209f, 1.906f, 2.609f, 5.351f}},    //  64 x 128, eight waves, two chunks per sub-step
+    {4, 2, 8, 4, 1, true, {1.034f, 2.290f, 3.605f, 4.644f, 8.583f}},    //  64 x 256, eight waves
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
-template<int TTILES, int NTW, int WAVES, int D>
+template<int TTILES, int NTW, int WAVES, int D, int KS>
 hipError_t launch_v(int splits, const GemmArgs& a, const Scratch& sc, hipStream_t st)
 {
     constexpr int TT = 16 * TTILES, TN = 16 * NTW * WAVES;
@@ -526,7 +546,7 @@ hipError_t launch_v(int splits, const GemmArgs& a, const Scratch& sc, hipStream_
     const u32x4_t* A4 = reinterpret_cast<const u32x4_t*>(a.A);
 #define W4A16_LAUNCH(EPI)                                                                                              \
     do {                                                                                                               \
-        auto       kfn = prefill_kernel<TTILES, NTW, WAVES, D, EPI>;                                                           \
+        auto       kfn = prefill_kernel<TTILES, NTW, WAVES, D, KS, EPI>;                                                           \
         hipError_t e   = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),                                       \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
         if (e != hipSuccess) return e;                                                                                 \
@@ -582,13 +602,13 @@ hipError_t prefill_launch(int v, int splits, const GemmArgs& a, const Scratch& s
 {
     if (splits > 1 && (sc.ws == nullptr || sc.cnt == nullptr)) return hipErrorInvalidValue;
     switch (v) {
-        case 0: return launch_v<8, 2, 8, 2>(splits, a, sc, st);
-        case 1: return launch_v<16, 2, 4, 2>(splits, a, sc, st);
-        case 2: return launch_v<8, 2, 4, 2>(splits, a, sc, st);
-        case 3: return launch_v<4, 2, 4, 4>(splits, a, sc, st);
-        case 4: return launch_v<4, 1, 4, 4>(splits, a, sc, st);
-        case 5: return launch_v<4, 1, 8, 4>(splits, a, sc, st);
-        default: return launch_v<4, 2, 8, 4>(splits, a, sc, st);
+        case 0: return launch_v<8, 2, 8, 2, 1>(splits, a, sc, st);
+        case 1: return launch_v<16, 2, 4, 2, 1>(splits, a, sc, st);
+        case 2: return launch_v<8, 2, 4, 2, 1>(splits, a, sc, st);
+        case 3: return launch_v<4, 2, 4, 4, 1>(splits, a, sc, st);
+        case 4: return launch_v<4, 1, 4, 4, 2>(splits, a, sc, st);
+        case 5: return launch_v<4, 1, 8, 4, 2>(splits, a, sc, st);
+        default: return launch_v<4, 2, 8, 4, 1>(splits, a, sc, st);
     }
 }
 
