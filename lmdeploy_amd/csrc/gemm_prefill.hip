@@ -7,15 +7,15 @@
 // tiled layout IS the MFMA operand layout), dequantises them to the reference's exact fp16
 // weight fp16_rn((q - z) * s) and uses them as the A operand of v_mfma_f32_16x16x32_f16.
 // The activations of the tile go from global memory directly into LDS (no registers, no
-// ds_write), double buffered, one 128-wide K step per quantisation group, and are read as the
-// B operand by all four waves, so no weight is dequantised twice and no activation is fetched
+// ds_write), D buffers deep, one 128-wide K step per quantisation group, and are read as the
+// B operand by all waves, so no weight is dequantised twice and no activation is fetched
 // twice per workgroup.  With weights as A the accumulator of a lane holds four adjacent
 // features of one token, which makes every epilogue (plain, SiLU-gate on feature pairs,
 // residual add) lane-local.
 //
 // The K loop is one hand-scheduled instruction stream per wave: every MFMA is followed by its
-// share of the NEXT k32 step's dequantisation, LDS fragment reads and global loads, so that a
-// single wave keeps the matrix pipe busy while it issues everything else (measured on this
+// share of the NEXT sub-step's (one or two k32 chunks) dequantisation, LDS fragment reads and
+// global loads, so that a single wave keeps the matrix pipe busy while it issues everything else (measured on this
 // part: an MFMA occupies the pipe for 16 cycles and issues in 4; two vector instructions fit
 // behind each one for free, a third does not).  The MFMAs are inline assembly with the
 // accumulators tied in place in AGPRs; loads are inline assembly waited for by count.
@@ -85,7 +85,7 @@ __device__ __forceinline__ void wait_vm(V& v)
 // LDS fragment read from inline assembly (byte address + immediate), and its wait.  Left to the
 // compiler, each activation fragment was read right before the MFMAs that use it, which then
 // waited a full LDS latency; and any compiler-visible LDS read after a direct-to-LDS load would
-// be preceded by a wait for ALL loads in flight.  Here the fragments of a k32 step are requested
+// be preceded by a wait for ALL loads in flight.  Here the fragments of a sub-step are requested
 // during the previous one.
 template<int OFF>
 __device__ __forceinline__ void lds_read128(half8_t& dst, uint32_t addr)
@@ -246,8 +246,8 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
 
-    // State carried from one k32 step to the next (and across K steps): dequantised weights and
-    // activation fragments of the current / next k32 step, zero points and scale of the current /
+    // State carried from one sub-step to the next (and across K steps): dequantised weights and
+    // activation fragments of the current / next sub-step, zero points and scale of the current /
     // next group.
     half8_t wf[2][KS][NTW];   // [sub-step parity][chunk][tile]
     half8_t xf[2][KS][TTILES];
@@ -263,7 +263,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         }
     };
     // The dequantisation of word J of every tile of `w`, as 13 * NTW single vector instructions
-    // (op = NTW * k + nt) so that they can be dealt out between the MFMAs of a k32 step:
+    // (op = NTW * k + nt) so that they can be dealt out between the MFMAs of a sub-step:
     // k = 0: w >> 8;  1..4: (w & mask) | magic;  5..8: - (offset + zero);  9..12: * scale.
     uint32_t dq[NTW][5];
     auto dequant_op = [&](auto P, auto J, auto OP, u32x4_t (&ws_)[NTW]) {
@@ -401,7 +401,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     }
     // no load may still be writing LDS or registers when the wave ends
     static_for<0, D>([&](auto dc) { wait_stage(I0{}, w[decltype(dc)::value], q[decltype(dc)::value]); });
-    // The last k32 step requested activation fragments for a step that does not exist.  Nothing
+    // The last sub-step requested activation fragments for a step that does not exist.  Nothing
     // reads them, so the compiler may hand their registers out again at once while the LDS reads
     // are still on their way and would land on the new owner: wait for them first.  (Tying the
     // registers to the wait would keep both fragment sets alive and cost registers in the loop;
