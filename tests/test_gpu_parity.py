@@ -371,6 +371,24 @@ def test_default_dispatch_over_token_counts(tm, gemm, K, N):
             assert np.isfinite(got).all() and err <= TOL, (K, N, kind, T, gemm.pick(N, T, K), err)
 
 
+@pytest.mark.parametrize("kind", [0, 1, 2])
+def test_token_tails_of_the_reference_test(tm, gemm, kind):
+    """The token counts that the reference's mixed-GEMM test sweeps
+    (tests/csrc/gemm_dequantize/th_gemm_dequantize.py:170: 256, 177, 195, 125, 66, 33, 8, 2, 1) plus a few
+    odd ones, through the default dispatch, all three epilogues."""
+    K, N = 1024, 1024
+    Ts = (1, 2, 3, 7, 8, 9, 17, 33, 66, 125, 177, 195, 256)
+    d = O.make_inputs(1700 + kind, max(Ts), K, N, residual=True)
+    A, Q = convert(tm, d, N, K)
+    W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], 128)
+    for T in Ts:
+        dd = dict(d, X=d["X"][:T], R=d["R"][:T])
+        want = O.epilogue(O.gemm_acc(dd["X"], W), kind, dd["R"] if kind == 2 else None)
+        got = run(tm, gemm, dd, A, Q, T, K, N, kind)
+        err = O.max_abs_rel(got, want)
+        assert np.isfinite(got).all() and err <= TOL, (kind, T, gemm.pick(N, T, K), err)
+
+
 def test_ffn_block(tm, gemm):
     """LlamaFfnLayer's int4 branch as one call: fused gate/up + SiLU into the gating buffer, then w2
     (+ residual, in place), against the oracle chained through the same fp16 intermediate."""
