@@ -46,7 +46,7 @@ typedef struct w4a16_metric {
     int   kind;        /* 0 = decode kernel (column blocks), 1 = MFMA prefill kernel, 2 = decode kernel (strips) */
     int   tile_n;      /* output features per workgroup                         */
     int   tile_t;      /* tokens per workgroup                                  */
-    int   slices;      /* decode: K slices (wave groups) per workgroup            */
+    int   slices;      /* decode: K slices (wave groups) per workgroup; prefill: workgroups that split K */
     int   grid;        /* workgroups launched                                   */
     float ms;          /* total time of `count` launches, +inf if not feasible  */
     int   count;       /* number of timed launches                              */
