@@ -39,6 +39,7 @@ TRAFFIC_PREFILL_GATE_UP = 565.2e6
 LAYER_7B = [("qkv", 4096, 12288, 0), ("o", 4096, 4096, 0), ("gate_up", 4096, 22016, 1), ("down", 11008, 4096, 2)]
 DECODE_T = (1, 4, 8, 16)
 PREFILL_T = 2048
+BATCHED_T = (32, 64, 128, 256)   # reported per shape, outside the headline metric
 GROUP = 128
 
 
@@ -198,6 +199,15 @@ def main():
                 per_shape.append({"shape": name, "T": T, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
                                   "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 3)})
 
+    # ---- batched decode / short prompts: 32 .. 256 tokens (not part of `value`) ----------------
+    batched = []
+    if not args.no_per_shape:
+        for name, K, N, epi in LAYER_7B:
+            for T in BATCHED_T:
+                us = per_launch_us(name, (T,), passes=2)
+                batched.append({"shape": name, "T": T, "us": round(us, 2), "TFLOPs": round(flops(T, K, N) / us / 1e6, 1),
+                                "GBps": round(algorithmic_bytes(T, K, N, epi) / us / 1e3, 1)})
+
     # ---- prefill: T = 2048 ---------------------------------------------------------------------
     prefill = None
     if not args.no_prefill:
@@ -303,7 +313,8 @@ def main():
                    "launch": "eager" if args.eager else "hipgraph replay of one step",
                    "bytes_per_step": step_bytes},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-        "roofline": roofline, "cpu_baseline": cpu, "decode_per_shape": per_shape, "prefill": prefill,
+        "roofline": roofline, "cpu_baseline": cpu, "decode_per_shape": per_shape, "batched_decode_per_shape": batched,
+        "prefill": prefill,
         "layers32_m8": layers32, "library_ceilings": ceilings,
     }
     print(json.dumps(line))
