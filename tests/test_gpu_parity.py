@@ -389,6 +389,42 @@ def test_token_tails_of_the_reference_test(tm, gemm, kind):
         assert np.isfinite(got).all() and err <= TOL, (kind, T, gemm.pick(N, T, K), err)
 
 
+def test_random_shapes_every_kernel(tm, gemm):
+    """Seeded random (K, N, T) x every kernel configuration x every epilogue, against an fp32 torch matmul on
+    the library's own dequantised weights (which test_dequantised_weights_bit_exact pins to the oracle)."""
+    import random
+    rng = random.Random(5)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7)
+    ran = 0
+    for case in range(24):
+        K, N = 128 * rng.randint(1, 44), 64 * rng.randint(1, 40)
+        T = rng.choice([1, 2, 5, 8, 13, 16, 17, 20, 31, 32, 33, 47, 64, 65, 100, 128, 129, 200, 257])
+        G = K // 128
+        qw = torch.randint(-2**31, 2**31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=gen)
+        qz = torch.randint(-2**31, 2**31 - 1, (G, N // 8), dtype=torch.int32, device="cuda", generator=gen)
+        s = (torch.randn((G, N), device="cuda", generator=gen).abs() * 0.01 + 1e-3).half()
+        A, Q = torch.empty_like(qw), torch.empty((G, N), dtype=torch.int32, device="cuda")
+        tm.convert_s4_k_m8(A, Q, s, qw, s, qz, N, K, 128)
+        W = tm.dequantize_repacked(A, Q, N, K).float()
+        X = torch.randn((T, K), device="cuda", generator=gen).half()
+        R = torch.randn((T, N), device="cuda", generator=gen).half()
+        y = (X.float() @ W).half().float()                       # the single rounding of the accumulator
+        want = {0: y, 1: y[:, 0::2] / (1 + torch.exp(-y[:, 0::2])) * y[:, 1::2], 2: R.float() + y}
+        for algo in [-1] + _algos(gemm):
+            for kind in (0, 1, 2):
+                C = torch.full((T, N // 2 if kind == 1 else N), float("nan"), dtype=torch.float16, device="cuda")
+                try:
+                    gemm.Run(C, A, X, Q, N, T, K, 128, kind, algo, residual=R if kind == 2 else None)
+                except tm.W4A16Error as e:
+                    assert e.code == -2, e
+                    continue
+                err = ((C.float() - want[kind]).abs().max() / want[kind].abs().max()).item()
+                assert err <= TOL, (K, N, T, algo, kind, err)
+                ran += 1
+    assert ran >= 1000
+
+
 def test_ffn_block(tm, gemm):
     """LlamaFfnLayer's int4 branch as one call: fused gate/up + SiLU into the gating buffer, then w2
     (+ residual, in place), against the oracle chained through the same fp16 intermediate."""
