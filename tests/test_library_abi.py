@@ -97,3 +97,15 @@ def test_product_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".cpp", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, "%s mentions the oracle" % f
+
+
+def test_build_module_imports_without_the_library():
+    """`python -m lmdeploy_amd.build` must work in a fresh checkout: importing the package or its build
+    module must not need (or load) the shared library."""
+    import subprocess
+    import sys
+    code = ("import sys, lmdeploy_amd, lmdeploy_amd.build; "
+            "assert 'lmdeploy_amd._lib' not in sys.modules and 'lmdeploy_amd.turbomind' not in sys.modules")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
