@@ -270,7 +270,7 @@ def main():
         import numpy as np
         from oracle import w4a16_oracle as O
         T, reps = 8, 5
-        t_deq = t_mm = 0.0
+        t_deq = t_mm = t_mm1 = 0.0
         by = 0
         for i, (name, K, N, epi) in enumerate(LAYER_7B):
             d = O.make_inputs(77 + i, T, K, N, GROUP, residual=(epi == 2))
@@ -286,11 +286,17 @@ def main():
             t_deq += sorted(deq)[reps // 2]
             t_mm += sorted(mm)[reps // 2]
             by += algorithmic_bytes(T, K, N, epi)
+            nthreads = torch.get_num_threads()   # the same matmul once on a single thread, for scale
+            torch.set_num_threads(1)
+            t1 = time.perf_counter()
+            O.epilogue(O.gemm_acc(d["X"], W), epi, d.get("R"))
+            t_mm1 += time.perf_counter() - t1
+            torch.set_num_threads(nthreads)
         cpu = {"value": round(by / (t_deq + t_mm) / 1e9, 4), "unit": "GB/s", "cores": torch.get_num_threads(),
                "kind": "port", "host_cpus": os.cpu_count(),
                "sample": "one Llama-2-7B layer (qkv, o, gate_up+SiLU, down+residual) at T=8, median of %d passes per "
                          "GEMM: numpy unpack+dequantise %.2f s (1 thread) + torch fp32 matmul+epilogue %.3f s "
-                         "(%d threads)" % (reps, t_deq, t_mm, torch.get_num_threads())}
+                         "(%d threads; %.3f s on 1 thread)" % (reps, t_deq, t_mm, torch.get_num_threads(), t_mm1)}
 
     # ---- the full 32-layer GEMM sequence of one decode step at M = 8 (every layer its own weights) ----
     seq_T = 8
