@@ -156,10 +156,57 @@ def _mfma_hazards(name: str, lines: List[Tuple[int, str]]) -> List[str]:
             in_asm = False
             continue
         code = raw.split(";")[0].strip()
-        if not code or code.startswith(".") or code.endswith(":"):
+        if not code or (code.startswith(".") and not code.endswith(":")):
             continue
-        seq.append((ln, code, in_asm))
+        seq.append((ln, code, in_asm))  # (labels stay in the sequence: they delimit loops)
     out = []
+    # A loop whose body holds inline-assembly MFMAs must not move accumulators at all: across the
+    # back edge the MFMAs at the bottom of the body precede whatever stands at its top.  Blocks and
+    # edges of the function; a branch back to a label closes a loop only if the branch can be
+    # reached from that label (out-of-line blocks at the end of a function also jump backwards).
+    starts = sorted({0} | {k for k, (_, c, _) in enumerate(seq) if c.endswith(":")}
+                    | {k + 1 for k, (_, c, _) in enumerate(seq) if _BRANCH.match(c) or c.startswith("s_endpgm")})
+    starts = [k for k in starts if k < len(seq)]
+    block_of = {}
+    for bi, k0 in enumerate(starts):
+        for k in range(k0, starts[bi + 1] if bi + 1 < len(starts) else len(seq)):
+            block_of[k] = bi
+    label_block = {c[:-1]: block_of[k] for k, (_, c, _) in enumerate(seq) if c.endswith(":")}
+    succ = [set() for _ in starts]
+    for bi, k0 in enumerate(starts):
+        k1 = (starts[bi + 1] if bi + 1 < len(starts) else len(seq)) - 1
+        last = seq[k1][1]
+        m = _BRANCH.match(last)
+        if m and m.group(2) in label_block:
+            succ[bi].add(label_block[m.group(2)])
+        if not last.startswith("s_endpgm") and not (m and m.group(1) == "branch") and bi + 1 < len(starts):
+            succ[bi].add(bi + 1)
+
+    def reach(src, edges):
+        seen, work = {src}, [src]
+        while work:
+            for nb in edges[work.pop()]:
+                if nb not in seen:
+                    seen.add(nb)
+                    work.append(nb)
+        return seen
+
+    pred = [set() for _ in starts]
+    for bi, ss in enumerate(succ):
+        for t in ss:
+            pred[t].add(bi)
+    for bi in range(len(starts)):
+        for h in succ[bi]:
+            if h > bi or bi not in reach(h, succ):
+                continue  # not a back edge of a loop
+            body = reach(h, succ) & reach(bi, pred)
+            ks = [k for k in range(len(seq)) if block_of[k] in body]
+            if any(seq[k][2] and _MFMA.match(seq[k][1]) for k in ks):
+                for k in ks:
+                    bl, bc, ba = seq[k]
+                    if not ba and bc.startswith("v_accvgpr"):
+                        out.append("%s: line %d moves an accumulator inside a loop of inline-assembly MFMAs: %s"
+                                   % (name, bl, bc))
     for k, (ln, code, asm) in enumerate(seq):
         if asm or not code.startswith("v_accvgpr"):
             continue
@@ -175,11 +222,12 @@ def _mfma_hazards(name: str, lines: List[Tuple[int, str]]) -> List[str]:
                            % (name, ln, waited, pl, code))
                 break
             n = _NOP.match(pc)
-            waited += int(n.group(1)) + 1 if n else 1
+            if not pc.endswith(":"):
+                waited += int(n.group(1)) + 1 if n else 1
             j -= 1
         if code.startswith("v_accvgpr_write") or code.startswith("v_accvgpr_mov"):
             dst = next(iter(_regs(_AREG.search(code))))
-            for pl, pc, pasm in seq[k + 1:k + 3]:
+            for pl, pc, pasm in [x for x in seq[k + 1:k + 6] if not x[1].endswith(":")][:2]:
                 m = _MFMA.match(pc) if pasm else None
                 if m and dst in {r for a in _AREG.finditer(m.group(3)) for r in _regs(a)}:
                     out.append("%s: line %d writes a%d right before the MFMA of line %d reads it: %s"

@@ -59,3 +59,25 @@ def test_parking_an_in_flight_register_in_an_agpr_is_reported():
 def test_parking_a_settled_register_is_accepted():
     asm = HEAD + load(48) + "\ts_waitcnt vmcnt(0)\n\tv_accvgpr_write_b32 a106, v51\n" + TAIL
     assert lint(asm) == []
+
+
+def mfma(acc):
+    return "\t;;#ASMSTART\n\tv_mfma_f32_16x16x32_f16 a[%d:%d], v[0:3], v[4:7], a[%d:%d]\n\t;;#ASMEND\n" % (acc, acc + 3, acc, acc + 3)
+
+
+def test_accumulator_read_right_after_an_inline_mfma_is_reported():
+    asm = HEAD + mfma(8) + "\tv_accvgpr_read_b32 v20, a9\n" + TAIL
+    msgs = lint(asm)
+    assert len(msgs) == 1 and "wait states" in msgs[0]
+
+
+def test_accumulator_read_after_the_pipe_has_drained_is_accepted():
+    asm = HEAD + mfma(8) + "\t;;#ASMSTART\n\ts_nop 15\n\ts_nop 15\n\t;;#ASMEND\n\tv_accvgpr_read_b32 v20, a9\n" + TAIL
+    assert lint(asm) == []
+
+
+def test_accumulator_move_inside_a_loop_of_inline_mfmas_is_reported():
+    # at the top of the body, textually before the MFMA, but reached again across the back edge
+    asm = (HEAD + ".LBB0_1:\n\tv_accvgpr_mov_b32 a8, a12\n" + mfma(8) + "\ts_cbranch_scc1 .LBB0_1\n" + TAIL)
+    msgs = lint(asm)
+    assert any("inside a loop" in m for m in msgs)
