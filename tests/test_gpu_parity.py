@@ -389,6 +389,31 @@ def test_token_tails_of_the_reference_test(tm, gemm, kind):
         assert np.isfinite(got).all() and err <= TOL, (kind, T, gemm.pick(N, T, K), err)
 
 
+def test_every_kernel_is_deterministic(tm, gemm):
+    """Sliced and split K sums are added in a fixed order (as the reference's sum_slices, gemm_template.h:288-333),
+    so repeated launches must agree bit for bit, whichever workgroup happens to arrive last."""
+    K, N, T = 4224, 1024, 100
+    d = O.make_inputs(4242, T, K, N, residual=True)
+    A, Q = convert(tm, d, N, K)
+    X, R = dev(d["X"]), dev(d["R"])
+    ran = 0
+    for algo in _algos(gemm):
+        first = None
+        for rep in range(8):
+            C = torch.full((T, N), float("nan"), dtype=torch.float16, device="cuda")
+            try:
+                gemm.Run(C, A, X, Q, N, T, K, 128, gemm.kFusedAdd, algo, residual=R)
+            except tm.W4A16Error:
+                break
+            got = C.view(torch.int16)
+            if first is None:
+                first = got.clone()
+            else:
+                assert torch.equal(got, first), (algo, rep)
+        ran += first is not None
+    assert ran >= 30
+
+
 def test_random_shapes_every_kernel(tm, gemm):
     """Seeded random (K, N, T) x every kernel configuration x every epilogue, against an fp32 torch matmul on
     the library's own dequantised weights (which test_dequantised_weights_bit_exact pins to the oracle)."""
