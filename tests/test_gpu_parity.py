@@ -389,6 +389,39 @@ def test_token_tails_of_the_reference_test(tm, gemm, kind):
         assert np.isfinite(got).all() and err <= TOL, (kind, T, gemm.pick(N, T, K), err)
 
 
+def test_graph_replays_of_kernels_that_use_the_handle_scratch(tm, gemm):
+    """The split-K kernels keep arrival counters in the handle and reset them themselves (no memset node).
+    A captured graph holding one GEMM per such kernel is replayed several times, with new activations
+    written eagerly between the replays, and every replay must equal the eager result bit for bit."""
+    K, N, T = 4224, 1024, 100
+    d = O.make_inputs(777, T, K, N, residual=True)
+    A, Q = convert(tm, d, N, K)
+    X, R = dev(d["X"]), dev(d["R"])
+    ms = gemm.Measure(torch.empty((T, N), dtype=torch.float16, device="cuda"), A, X, Q, N, T, K, 128, gemm.kGemm)
+    algos = [m.id for m in ms if m.feasible]           # every kernel that can run the shape, split-K ones included
+    assert sum(1 for m in ms if m.feasible and m.kind == 1 and m.slices > 1) >= 4
+    gemm.clear_tuning()
+    outs = [torch.empty((T, N), dtype=torch.float16, device="cuda") for _ in algos]
+    stream = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=stream):
+        st = torch.cuda.current_stream().cuda_stream
+        for a, C in zip(algos, outs):
+            gemm.Run(C, A, X, Q, N, T, K, 128, gemm.kFusedAdd, a, residual=R, stream=st)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(3)
+    for rep in range(5):
+        X.copy_(torch.randn((T, K), device="cuda", generator=gen).half())       # eager work between replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for a, C in zip(algos, outs):
+            E = torch.empty_like(C)
+            gemm.Run(E, A, X, Q, N, T, K, 128, gemm.kFusedAdd, a, residual=R)
+            torch.cuda.synchronize()
+            assert torch.equal(E.view(torch.int16), C.view(torch.int16)), (rep, a)
+
+
 def test_every_kernel_is_deterministic(tm, gemm):
     """Sliced and split K sums are added in a fixed order (as the reference's sum_slices, gemm_template.h:288-333),
     so repeated launches must agree bit for bit, whichever workgroup happens to arrive last."""
