@@ -30,6 +30,7 @@ extern "C" {
 #define W4A16_EHIP (-3)      /* the HIP runtime reported an error            */
 #define W4A16_EARG (-4)      /* null pointer / negative size / bad enum      */
 #define W4A16_EALGO (-5)     /* algo_id out of range                         */
+#define W4A16_ESCRATCH (-6)  /* the split-K scratch this launch needs is not available */
 
 /* epilogues; 0 and 1 are GemmS4F16::Type (gemm_s4_f16.h:23-27), 2 is an extension */
 #define W4A16_GEMM 0
@@ -53,9 +54,13 @@ typedef struct w4a16_metric {
 } w4a16_metric;
 
 /* GemmS4F16::GemmS4F16 / ~GemmS4F16 (gemm_s4_f16.h:19-21, gemm_s4_f16.cu:236-252).
- * The handle owns two events and a fixed 64 MiB scratch buffer for split-K partial sums
- * (plus arrival counters); it binds to the current device.  GEMMs issued through one
- * handle must be ordered on one stream at a time, because they share that scratch. */
+ * The handle owns two events and 256 KiB of arrival counters; it binds to the current device.
+ * A fixed 64 MiB workspace for split-K partial sums is allocated by the first launch that splits K
+ * (some shapes between 17 and 512 tokens, narrow matrices at up to 16) and kept until
+ * w4a16_destroy.  That first launch must not be under graph capture: there, a handle that has no
+ * workspace yet uses kernels that need none (algo_id < 0) or fails with W4A16_ESCRATCH (explicit
+ * algo_id).  GEMMs issued through one handle must be ordered on one stream at a time, because they
+ * share that scratch. */
 int  w4a16_create(w4a16_handle** out);
 void w4a16_destroy(w4a16_handle* h);
 
@@ -73,7 +78,15 @@ void w4a16_destroy(w4a16_handle* h);
  *                         (no counterpart in GemmS4F16; the add of
  *                          llama_decoder_kernels.cu:52-57 applied as in LlamaDecoder.cc:228-235)
  * algo_id < 0 selects a kernel by heuristic (gemm_s4_f16.cu:184-206 `Estimate`).
- * Requires group_size == 128, k % 128 == 0, n_out % 16 == 0, tokens >= 0. */
+ * Requires group_size == 128, k % 128 == 0, n_out % 16 == 0, tokens >= 0; A and X aligned to 16
+ * bytes, Q to 4, C and R to 4 (to 8 when an MFMA prefill kernel runs, i.e. above 32 tokens, except
+ * for W4A16_FUSED_SILU_FFN).
+ * Numerics: the kernels for up to 32 tokens (and narrow matrices up to ~128) scale each group's
+ * fp32 partial sum by the fp16 scale; the MFMA prefill kernels multiply by the fp16 weight
+ * fp16((q - z) * s), without the reference's flush of subnormal products to zero (common.h:229-230
+ * mul.ftz; only w4a16_dequantize_repacked flushes).  Both are within the 1e-2 tolerance of each
+ * other and of the reference, but not bit-identical: the same input can give different bits on the
+ * two sides of a hand-over point between kernel families. */
 int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R,
                int n_out, int tokens, int k, int group_size, int epilogue, int algo_id, void* stream);
 
@@ -90,9 +103,11 @@ int w4a16_ffn(w4a16_handle* h, void* ffn_output, void* gating_buf, const void* f
 
 /* GemmS4F16::Measure (gemm_s4_f16.h:29-39, gemm_s4_f16.cu:98-169): times every feasible
  * kernel (10 warm-up + 100 timed launches each) and writes up to `capacity` rows sorted
- * by time; returns the number of rows, or a negative error.  Synchronises `stream`.  The handle
- * remembers the fastest kernel for (n_out, tokens, k); later `w4a16_gemm` calls with algo_id < 0
- * and exactly that shape use it (see `w4a16_pick`). */
+ * by time; returns the number of rows, or a negative error.  Synchronises `stream` (so it cannot
+ * run under capture).  The handle remembers the fastest kernel for (n_out, tokens, k); later
+ * `w4a16_gemm` calls with algo_id < 0 and exactly that shape use it (see `w4a16_pick`).  Because
+ * kernel families round differently (see w4a16_gemm), a Measure call can change the low bits that
+ * later w4a16_gemm calls of that shape return; `w4a16_clear_tuning` restores the heuristic. */
 int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R,
                   int n_out, int tokens, int k, int group_size, int epilogue,
                   w4a16_metric* metrics, int capacity, void* stream);

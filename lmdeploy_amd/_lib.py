@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # W4A16_LIB overrides the in-tree library (e.g. to try a differently tuned build)
 LIB_PATH = os.environ.get("W4A16_LIB") or os.path.join(_HERE, "lib", "libw4a16.so")
 
-OK, EGROUP, ESHAPE, EHIP, EARG, EALGO = 0, -1, -2, -3, -4, -5
+OK, EGROUP, ESHAPE, EHIP, EARG, EALGO, ESCRATCH = 0, -1, -2, -3, -4, -5, -6
 GEMM, FUSED_SILU_FFN, FUSED_ADD = 0, 1, 2
 
 

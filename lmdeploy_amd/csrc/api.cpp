@@ -36,6 +36,11 @@ bool aligned16(const void* p)
     return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }
 
+bool aligned8(const void* p)
+{
+    return (reinterpret_cast<uintptr_t>(p) & 7u) == 0;
+}
+
 }  // namespace
 
 struct w4a16_handle {
@@ -103,11 +108,20 @@ const Algo& algo_at(int id)
     return table()[id];
 }
 
-bool algo_feasible(int id, int N, int T, int K)
+bool algo_feasible(int id, int N, int T, int K, const Scratch& lim)
 {
     const Algo& a = algo_at(id);
     if (a.kind == 2) return strip_feasible(a.param, a.tile_t, N, T, K);
-    return a.kind == 0 ? decode_feasible(a.dc, N, T, K) : prefill_feasible(a.param, a.slices, N, T, K);
+    return a.kind == 0 ? decode_feasible(a.dc, N, T, K) :
+                         prefill_feasible(a.param, a.slices, N, T, K, lim.ws_bytes, lim.cnt_len);
+}
+
+size_t algo_scratch_bytes(int id, int N, int T, int K, const Scratch& lim)
+{
+    const Algo& a = algo_at(id);
+    if (a.kind == 2) return 0;
+    return a.kind == 0 ? decode_scratch_bytes(a.dc, N, T, K, lim.ws_bytes, lim.cnt_len) :
+                         prefill_scratch_bytes(a.param, a.slices, N, T, K);
 }
 
 int algo_grid(int id, int N, int T, int K, const Scratch& sc)
@@ -129,7 +143,7 @@ hipError_t algo_launch(int id, const GemmArgs& g, const Scratch& sc, hipStream_t
 // every MFMA prefill tile, unsplit and with K split 2, 4 or 8 ways, is priced with a model of
 // measured step times, and so is the decode kernel (which re-reads the weights once per 16
 // tokens); the cheapest wins.  Up to 16 tokens: the decode kernel, see below.
-int algo_pick(int N, int T, int K)
+int algo_pick(int N, int T, int K, const Scratch& lim)
 {
     if (T <= 0 || N <= 0 || K <= 0) return -1;
     if (T > 16) {
@@ -137,7 +151,7 @@ int algo_pick(int N, int T, int K)
         double best_us = 0;
         for (int id = 0; id < algo_count(); ++id) {
             const Algo& a = algo_at(id);
-            if (a.kind != 1 || !algo_feasible(id, N, T, K)) continue;
+            if (a.kind != 1 || !algo_feasible(id, N, T, K, lim)) continue;
             const double us = prefill_estimate_us(a.param, a.slices, N, T, K);
             if (best < 0 || us < best_us) best = id, best_us = us;
         }
@@ -153,7 +167,7 @@ int algo_pick(int N, int T, int K)
         if (T <= 32) {
             for (int id = 0; id < algo_count() && strip32 < 0; ++id) {
                 const Algo& a = algo_at(id);
-                if (a.kind == 2 && a.tile_t == 32 && a.param == 1 && algo_feasible(id, N, T, K)) strip32 = id;
+                if (a.kind == 2 && a.tile_t == 32 && a.param == 1 && algo_feasible(id, N, T, K, lim)) strip32 = id;
             }
             strip32_us = 3.0 + (1.25 + 0.35 * (T - 16) / 16.0) * ((double)K * N / 2) / 4.2e6;
         }
@@ -172,7 +186,7 @@ int algo_pick(int N, int T, int K)
         for (int per_cu : {want, 1}) {
             for (int id = 0; id < algo_count(); ++id) {
                 const Algo& a = algo_at(id);
-                if (a.kind == 2 && a.tile_t == 16 && a.param == per_cu && algo_feasible(id, N, T, K)) return id;
+                if (a.kind == 2 && a.tile_t == 16 && a.param == per_cu && algo_feasible(id, N, T, K, lim)) return id;
             }
         }
     }
@@ -198,11 +212,11 @@ int algo_pick(int N, int T, int K)
     for (int id = 0; id < algo_count(); ++id) {
         const Algo& a = algo_at(id);
         if (a.kind == 0 && a.dc.r == 1 && a.dc.depth == 4 && a.dc.wn == wn && a.dc.sk == sk && a.dc.fill == fill &&
-            algo_feasible(id, N, T, K))
+            algo_feasible(id, N, T, K, lim))
             return id;
     }
     for (int id = 0; id < algo_count(); ++id)
-        if (algo_feasible(id, N, T, K)) return id;
+        if (algo_feasible(id, N, T, K, lim)) return id;
     return -1;
 }
 
@@ -212,10 +226,10 @@ using namespace w4a16;
 
 namespace {
 
-int check_gemm_args(const w4a16_handle* h, const void* C, const void* A, const void* X, const void* Q,
-                    const void* R, int n_out, int tokens, int k, int group_size, int epilogue)
+// Validates the arguments of a GEMM without touching the GPU: < 0 error, 1 nothing to do, 0 go on.
+int check_gemm_args(const void* C, const void* A, const void* X, const void* Q, const void* R, int n_out, int tokens,
+                    int k, int group_size, int epilogue)
 {
-    if (!h) return fail(W4A16_EARG, "null handle");
     if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
     if (epilogue < W4A16_GEMM || epilogue > W4A16_FUSED_ADD) return fail(W4A16_EARG, "unknown epilogue %d", epilogue);
     if (n_out < 0 || tokens < 0 || k < 0) return fail(W4A16_EARG, "negative size");
@@ -226,7 +240,15 @@ int check_gemm_args(const w4a16_handle* h, const void* C, const void* A, const v
         (reinterpret_cast<uintptr_t>(Q) & 3u) || (R && (reinterpret_cast<uintptr_t>(R) & 3u)))
         return fail(W4A16_EARG, "misaligned pointer (A and X need 16 bytes, C, Q, R need 4)");
     if (k == 0 || k % 128 != 0 || n_out % 16 != 0) return fail(W4A16_ESHAPE, "no feasible kernel found");
-    (void)hipGetLastError();  // an error some earlier caller left behind is not this launch's
+    return 0;
+}
+
+// The MFMA prefill kernels store (and read the residual) four features at a time.
+int check_prefill_alignment(int algo_id, const void* C, const void* R, int epilogue)
+{
+    if (algo_at(algo_id).kind != 1 || epilogue == W4A16_FUSED_SILU_FFN) return 0;
+    if (!aligned8(C) || (R && !aligned8(R)))
+        return fail(W4A16_EARG, "misaligned pointer (C and R need 8 bytes for more than 32 tokens)");
     return 0;
 }
 
@@ -234,8 +256,34 @@ int check_gemm_args(const w4a16_handle* h, const void* C, const void* A, const v
 int pick_for(const w4a16_handle* h, int n_out, int tokens, int k)
 {
     const auto it = h->tuned.find(std::make_tuple(n_out, tokens, k));
-    if (it != h->tuned.end() && algo_feasible(it->second, n_out, tokens, k)) return it->second;
-    return algo_pick(n_out, tokens, k);
+    if (it != h->tuned.end() && algo_feasible(it->second, n_out, tokens, k, h->scratch)) return it->second;
+    return algo_pick(n_out, tokens, k, h->scratch);
+}
+
+// The partial-tile workspace of a handle is allocated when a launch first needs it.  That cannot
+// happen while `st` is being captured into a graph; `*have` then stays false.
+int ensure_workspace(w4a16_handle* h, hipStream_t st, bool* have)
+{
+    *have = h->scratch.ws != nullptr;
+    if (*have) return W4A16_OK;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) return W4A16_OK;
+    const hipError_t e = hipMalloc((void**)&h->scratch.ws, kWorkspaceBytes);
+    if (e != hipSuccess) {
+        h->scratch.ws = nullptr;
+        return hip_fail(e, "w4a16: allocating the split-K workspace");
+    }
+    *have = true;
+    return W4A16_OK;
+}
+
+// what an algo may use of a scratch that has no workspace yet: nothing
+Scratch without_workspace(const Scratch& sc)
+{
+    Scratch s = sc;
+    s.ws       = nullptr;
+    s.ws_bytes = 0;
+    return s;
 }
 
 }  // namespace
@@ -250,18 +298,17 @@ int w4a16_create(w4a16_handle** out)
     hipError_t e = hipGetDevice(&h->device);
     if (e == hipSuccess) e = hipEventCreate(&h->ev_start);
     if (e == hipSuccess) e = hipEventCreate(&h->ev_end);
-    if (e == hipSuccess) e = hipMalloc((void**)&h->scratch.ws, kWorkspaceBytes);
     if (e == hipSuccess) e = hipMalloc((void**)&h->scratch.cnt, kCounters * sizeof(int));
     if (e == hipSuccess) e = hipMemset(h->scratch.cnt, 0, kCounters * sizeof(int));
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
         if (h->ev_start) (void)hipEventDestroy(h->ev_start);
         if (h->ev_end) (void)hipEventDestroy(h->ev_end);
-        if (h->scratch.ws) (void)hipFree(h->scratch.ws);
         if (h->scratch.cnt) (void)hipFree(h->scratch.cnt);
         delete h;
         return hip_fail(e, "w4a16_create");
     }
+    h->scratch.ws       = nullptr;  // 64 MiB, allocated by the first launch that splits K (ensure_workspace)
     h->scratch.ws_bytes = kWorkspaceBytes;
     h->scratch.cnt_len  = kCounters;
     *out = h;
@@ -273,7 +320,7 @@ void w4a16_destroy(w4a16_handle* h)
     if (!h) return;
     (void)hipEventDestroy(h->ev_end);
     (void)hipEventDestroy(h->ev_start);
-    (void)hipFree(h->scratch.ws);
+    if (h->scratch.ws) (void)hipFree(h->scratch.ws);
     (void)hipFree(h->scratch.cnt);
     delete h;
 }
@@ -302,15 +349,33 @@ int w4a16_algo_count(void)
 int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R, int n_out,
                int tokens, int k, int group_size, int epilogue, int algo_id, void* stream)
 {
-    const int chk = check_gemm_args(h, C, A, X, Q, R, n_out, tokens, k, group_size, epilogue);
+    if (!h) return fail(W4A16_EARG, "null handle");
+    const int chk = check_gemm_args(C, A, X, Q, R, n_out, tokens, k, group_size, epilogue);
     if (chk < 0) return chk;
     if (chk > 0) return W4A16_OK;
     if (algo_id >= algo_count()) return fail(W4A16_EALGO, "algo_id %d out of range (0..%d)", algo_id, algo_count() - 1);
-    if (algo_id < 0) algo_id = pick_for(h, n_out, tokens, k);
-    if (algo_id < 0 || !algo_feasible(algo_id, n_out, tokens, k)) return fail(W4A16_ESHAPE, "no feasible kernel found");
+    const bool chosen = algo_id >= 0;
+    if (!chosen) algo_id = pick_for(h, n_out, tokens, k);
+    if (algo_id < 0 || !algo_feasible(algo_id, n_out, tokens, k, h->scratch))
+        return fail(W4A16_ESHAPE, "no feasible kernel found");
+    Scratch sc = h->scratch;
+    if (algo_scratch_bytes(algo_id, n_out, tokens, k, sc) > 0) {
+        bool have = false;
+        if (int rc = ensure_workspace(h, (hipStream_t)stream, &have)) return rc;
+        sc = h->scratch;
+        if (!have) {
+            // the stream is being captured and this handle has never split K before: nothing can be allocated now
+            sc = without_workspace(sc);
+            if (!chosen) algo_id = algo_pick(n_out, tokens, k, sc);
+            if (algo_id < 0 || !algo_feasible(algo_id, n_out, tokens, k, sc))
+                return fail(W4A16_ESCRATCH, "this kernel splits K through the handle's workspace, which cannot be "
+                                            "allocated while the stream is capturing: run the shape once before");
+        }
+    }
+    if (int rc = check_prefill_alignment(algo_id, C, R, epilogue)) return rc;
     GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
                n_out,        tokens,             k,                  epilogue};
-    const hipError_t e = algo_launch(algo_id, g, h->scratch, (hipStream_t)stream);
+    const hipError_t e = algo_launch(algo_id, g, sc, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "w4a16_gemm launch");
     return W4A16_OK;
 }
@@ -330,12 +395,17 @@ int w4a16_ffn(w4a16_handle* h, void* ffn_output, void* gating_buf, const void* f
 int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R, int n_out,
                   int tokens, int k, int group_size, int epilogue, w4a16_metric* metrics, int capacity, void* stream)
 {
-    const int chk = check_gemm_args(h, C, A, X, Q, R, n_out, tokens, k, group_size, epilogue);
+    if (!h) return fail(W4A16_EARG, "null handle");
+    const int chk = check_gemm_args(C, A, X, Q, R, n_out, tokens, k, group_size, epilogue);
     if (chk < 0) return chk;
     if (!metrics || capacity <= 0) return fail(W4A16_EARG, "no room for metrics");
     if (chk > 0) return 0;
     constexpr int kWarmup = 10, kMeasure = 100;  // gemm_s4_f16.cu:258-259
     hipStream_t   st   = (hipStream_t)stream;
+    bool          have = false;
+    if (int rc = ensure_workspace(h, st, &have)) return rc;
+    if (!have) return fail(W4A16_EARG, "w4a16_measure synchronises: it cannot run on a capturing stream");
+    if (!aligned8(C) || (R && !aligned8(R))) return fail(W4A16_EARG, "misaligned pointer (w4a16_measure needs C and R aligned to 8 bytes)");
     const int     best = pick_for(h, n_out, tokens, k);
     GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
                n_out,        tokens,             k,                  epilogue};
@@ -349,7 +419,7 @@ int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const 
         m.tile_t   = a.tile_t;
         m.slices   = a.slices;
         m.best     = id == best;
-        m.feasible = algo_feasible(id, n_out, tokens, k);
+        m.feasible = algo_feasible(id, n_out, tokens, k, h->scratch);
         m.count    = 1;
         m.ms       = std::numeric_limits<float>::infinity();
         if (m.feasible) {
@@ -382,7 +452,6 @@ static int check_repack(const char* what, int m, int k, int m_mult, int k_mult)
     if (m < 0 || k < 0) return fail(W4A16_EARG, "%s: negative size", what);
     if (m % m_mult != 0 || k % k_mult != 0)
         return fail(W4A16_ESHAPE, "%s: m must be a multiple of %d and k of %d (got m=%d k=%d)", what, m_mult, k_mult, m, k);
-    (void)hipGetLastError();  // an error some earlier caller left behind is not this launch's
     return 0;
 }
 
@@ -475,7 +544,7 @@ const char* w4a16_last_error(void)
 
 const char* w4a16_version(void)
 {
-    return "w4a16-gfx950 0.1";
+    return "w4a16-gfx950 0.2";
 }
 
 }  // extern "C"

@@ -390,23 +390,18 @@ hipError_t launch_rtd(const DecodeParams& p, dim3 grid, dim3 block, size_t lds, 
     do {                                                                                                               \
         auto kfn = decode_kernel<R, TP, D, EPI>;                                                                       \
         if (lds > 64 * 1024) {                                                                                         \
-            static bool raised = false; /* per instantiation */                                                       \
-            if (!raised) {                                                                                             \
-                const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),                           \
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);    \
-                if (e != hipSuccess) return e;                                                                         \
-                raised = true;                                                                                         \
-            }                                                                                                          \
+            static std::atomic<uint64_t> raised{0}; /* per instantiation, one bit per device */                        \
+            const hipError_t e = raise_lds_limit(reinterpret_cast<const void*>(kfn), (int)kMaxLds, raised);            \
+            if (e != hipSuccess) return e;                                                                             \
         }                                                                                                              \
-        hipLaunchKernelGGL(kfn, grid, block, lds, st, p);                                                              \
+        return launch_kernel(kfn, grid, block, lds, st, p);                                                            \
     } while (0)
     switch (epilogue) {
-        case kEpiGemm: W4A16_LAUNCH(kEpiGemm); break;
-        case kEpiSilu: W4A16_LAUNCH(kEpiSilu); break;
-        default: W4A16_LAUNCH(kEpiAdd); break;
+        case kEpiGemm: W4A16_LAUNCH(kEpiGemm);
+        case kEpiSilu: W4A16_LAUNCH(kEpiSilu);
+        default: W4A16_LAUNCH(kEpiAdd);
     }
 #undef W4A16_LAUNCH
-    return hipGetLastError();
 }
 
 template<int R, int D>
@@ -465,6 +460,12 @@ bool decode_feasible(const DecodeConfig& cf, int N, int T, int K)
     if (cf.wn * cf.sk > kMaxWaves || cf.wn < 1 || cf.sk < 1 || (cf.wn & (cf.wn - 1)) != 0) return false;
     if (!((cf.r == 1 && (cf.depth == 4 || cf.depth == 8)) || (cf.r == 2 && cf.depth == 4))) return false;
     return make_plan(cf, N, T, K, 0, 0).ok;
+}
+
+size_t decode_scratch_bytes(const DecodeConfig& cf, int N, int T, int K, size_t ws_bytes, int cnt_len)
+{
+    const Plan pl = make_plan(cf, N, T, K, ws_bytes, cnt_len);
+    return pl.sk_wg > 1 ? (size_t)pl.z * pl.sk_wg * (N / kTileN) * 1024 : 0;
 }
 
 int decode_grid(const DecodeConfig& cf, int N, int T, int K, size_t ws_bytes, int cnt_len)

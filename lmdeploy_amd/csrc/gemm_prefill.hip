@@ -546,20 +546,19 @@ hipError_t launch_v(int splits, const GemmArgs& a, const Scratch& sc, hipStream_
     const u32x4_t* A4 = reinterpret_cast<const u32x4_t*>(a.A);
 #define W4A16_LAUNCH(EPI)                                                                                              \
     do {                                                                                                               \
-        auto       kfn = prefill_kernel<TTILES, NTW, WAVES, D, KS, EPI>;                                                           \
-        hipError_t e   = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),                                       \
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
+        auto                         kfn = prefill_kernel<TTILES, NTW, WAVES, D, KS, EPI>;                             \
+        static std::atomic<uint64_t> raised{0}; /* per instantiation, one bit per device */                            \
+        const hipError_t             e = raise_lds_limit(reinterpret_cast<const void*>(kfn), (int)lds, raised);        \
         if (e != hipSuccess) return e;                                                                                 \
-        hipLaunchKernelGGL(kfn, grid, block, lds, st, a.C, A4, a.X, a.Q, a.R, a.N, a.T, a.K, tiles_t, tiles_n,        \
-                           sc.ws, sc.cnt);                                                                             \
+        return launch_kernel(kfn, grid, block, lds, st, a.C, A4, a.X, a.Q, a.R, a.N, a.T, a.K, tiles_t, tiles_n,       \
+                             sc.ws, sc.cnt);                                                                           \
     } while (0)
     switch (a.epilogue) {
-        case kEpiGemm: W4A16_LAUNCH(kEpiGemm); break;
-        case kEpiSilu: W4A16_LAUNCH(kEpiSilu); break;
-        default: W4A16_LAUNCH(kEpiAdd); break;
+        case kEpiGemm: W4A16_LAUNCH(kEpiGemm);
+        case kEpiSilu: W4A16_LAUNCH(kEpiSilu);
+        default: W4A16_LAUNCH(kEpiAdd);
     }
 #undef W4A16_LAUNCH
-    return hipGetLastError();
 }
 
 }  // namespace
@@ -575,7 +574,15 @@ void prefill_tile(int v, int& tile_n, int& tile_t)
     tile_t = 16 * kVariants[v].ttiles;
 }
 
-bool prefill_feasible(int v, int splits, int N, int T, int K)
+size_t prefill_scratch_bytes(int v, int splits, int N, int T, int K)
+{
+    (void)K;
+    if (v < 0 || v >= kNumVariants || splits <= 1) return 0;
+    const int tn = 16 * kVariants[v].ntw * kVariants[v].waves, tt = 16 * kVariants[v].ttiles;
+    return (size_t)(N / tn) * ((T + tt - 1) / tt) * splits * tn * tt * 4;
+}
+
+bool prefill_feasible(int v, int splits, int N, int T, int K, size_t ws_bytes, int cnt_len)
 {
     if (v < 0 || v >= kNumVariants || N <= 0 || T <= 0 || K <= 0 || splits < 1) return false;
     const int tn = 16 * kVariants[v].ntw * kVariants[v].waves, tt = 16 * kVariants[v].ttiles;
@@ -586,7 +593,7 @@ bool prefill_feasible(int v, int splits, int N, int T, int K)
     if (splits > 1) {
         // at least two groups per split; partial tiles and counters must fit the handle's scratch
         if (K / kGroup < 2 * splits || splits > 65535) return false;
-        if (grid * splits * tn * tt * 4 > (int64_t)kWorkspaceBytes || grid > kCounters) return false;
+        if (grid * splits * tn * tt * 4 > (int64_t)ws_bytes || grid > cnt_len) return false;
     }
     return grid * splits < (1ll << 31);
 }

@@ -357,11 +357,10 @@ hipError_t launch_rt(const StripParams& p, dim3 grid, size_t lds, int epilogue, 
 {
     const dim3 block(64 * kWaves);
     switch (epilogue) {
-        case kEpiGemm: hipLaunchKernelGGL((strip_kernel<RMAX, TP, kEpiGemm>), grid, block, lds, st, p); break;
-        case kEpiSilu: hipLaunchKernelGGL((strip_kernel<RMAX, TP, kEpiSilu>), grid, block, lds, st, p); break;
-        default: hipLaunchKernelGGL((strip_kernel<RMAX, TP, kEpiAdd>), grid, block, lds, st, p); break;
+        case kEpiGemm: return launch_kernel(strip_kernel<RMAX, TP, kEpiGemm>, grid, block, lds, st, p);
+        case kEpiSilu: return launch_kernel(strip_kernel<RMAX, TP, kEpiSilu>, grid, block, lds, st, p);
+        default: return launch_kernel(strip_kernel<RMAX, TP, kEpiAdd>, grid, block, lds, st, p);
     }
-    return hipGetLastError();
 }
 
 template<int RMAX>

@@ -237,11 +237,11 @@ hipError_t launch_convert(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* A_sr
     const int64_t words = (int64_t)m * k / 8;
     const int64_t qn    = (int64_t)(k / kGroup) * m;
     if (words == 0) return hipSuccess;
-    if (A_dst)
-        hipLaunchKernelGGL(repack_weights_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, A_dst, A_src, m, k);
-    if (Q_dst)
-        hipLaunchKernelGGL(merge_q_kernel, dim3(blocks_for(qn)), dim3(kThreads), 0, st, Q_dst, scales, qzeros, qn);
-    return hipGetLastError();
+    hipError_t e = hipSuccess;
+    if (A_dst) e = launch_kernel(repack_weights_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, A_dst, A_src, m, k);
+    if (Q_dst && e == hipSuccess)
+        e = launch_kernel(merge_q_kernel, dim3(blocks_for(qn)), dim3(kThreads), 0, st, Q_dst, scales, qzeros, qn);
+    return e;
 }
 
 hipError_t launch_unpack(uint32_t* qweight, uint32_t* qzeros, uint16_t* scales, const uint32_t* A,
@@ -250,11 +250,11 @@ hipError_t launch_unpack(uint32_t* qweight, uint32_t* qzeros, uint16_t* scales, 
     const int64_t words = (int64_t)m * k / 8;
     const int64_t qw    = (int64_t)(k / kGroup) * m / 8;
     if (words == 0) return hipSuccess;
-    if (qweight)
-        hipLaunchKernelGGL(unrepack_weights_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, qweight, A, m, k);
-    if (qzeros || scales)
-        hipLaunchKernelGGL(split_q_kernel, dim3(blocks_for(qw)), dim3(kThreads), 0, st, qzeros, scales, Q, qw);
-    return hipGetLastError();
+    hipError_t e = hipSuccess;
+    if (qweight) e = launch_kernel(unrepack_weights_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, qweight, A, m, k);
+    if ((qzeros || scales) && e == hipSuccess)
+        e = launch_kernel(split_q_kernel, dim3(blocks_for(qw)), dim3(kThreads), 0, st, qzeros, scales, Q, qw);
+    return e;
 }
 
 hipError_t launch_dequantize_repacked(uint16_t* W, const uint32_t* A, const uint32_t* Q, int m, int k,
@@ -262,41 +262,36 @@ hipError_t launch_dequantize_repacked(uint16_t* W, const uint32_t* A, const uint
 {
     const int64_t words = (int64_t)m * k / 8;
     if (words == 0) return hipSuccess;
-    hipLaunchKernelGGL(dequantize_repacked_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, W, A, Q, m, k);
-    return hipGetLastError();
+    return launch_kernel(dequantize_repacked_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, W, A, Q, m, k);
 }
 
 hipError_t launch_dequantize_s4(void* dst, const uint32_t* src, size_t count, hipStream_t st)
 {
     if (count == 0) return hipSuccess;
-    hipLaunchKernelGGL(dequantize_s4_kernel, dim3(blocks_for((int64_t)count)), dim3(kThreads), 0, st, (uint4*)dst,
-                       src, (int64_t)count);
-    return hipGetLastError();
+    return launch_kernel(dequantize_s4_kernel, dim3(blocks_for((int64_t)count)), dim3(kThreads), 0, st, (uint4*)dst,
+                         src, (int64_t)count);
 }
 
 hipError_t launch_fuse_w1_w3(uint32_t* dst, const uint32_t* src, int m, int k, hipStream_t st)
 {
     const int64_t words = (int64_t)k * (2 * m / 8);
     if (words == 0) return hipSuccess;
-    hipLaunchKernelGGL(fuse_w1_w3_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, dst, src, m, k);
-    return hipGetLastError();
+    return launch_kernel(fuse_w1_w3_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, dst, src, m, k);
 }
 
 hipError_t launch_transpose_qk(uint32_t* dst, const uint32_t* src, int m, int k, int size_per_head, hipStream_t st)
 {
     const int64_t words = (int64_t)k * (m / 8);
     if (words == 0) return hipSuccess;
-    hipLaunchKernelGGL(transpose_qk_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, dst, src, m, k,
-                       size_per_head);
-    return hipGetLastError();
+    return launch_kernel(transpose_qk_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, dst, src, m, k,
+                         size_per_head);
 }
 
 hipError_t launch_from_reference(uint32_t* dst, const uint32_t* ref, int m, int k, hipStream_t st)
 {
     const int64_t words = (int64_t)m * k / 8;
     if (words == 0) return hipSuccess;
-    hipLaunchKernelGGL(from_reference_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, dst, ref, m, k);
-    return hipGetLastError();
+    return launch_kernel(from_reference_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, dst, ref, m, k);
 }
 
 }  // namespace w4a16

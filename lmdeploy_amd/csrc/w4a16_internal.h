@@ -1,8 +1,11 @@
-// Internal C++ interface between the C ABI (api.hip) and the kernel launchers.
+// Internal C++ interface between the C ABI (api.cpp) and the kernel launchers.
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <atomic>
+#include <tuple>
 
 namespace w4a16 {
 
@@ -35,8 +38,10 @@ struct Algo {
     DecodeConfig dc;       // decode only
 };
 
-// Scratch owned by a handle: split-K partial tiles and arrival counters.  Every handle has exactly
-// this much, so feasibility of a split-K launch does not depend on the handle.
+// Scratch of the split-K kernels: fp32 partial tiles and arrival counters.  A handle's scratch has
+// exactly this size (the partial tiles are allocated on first need, the counters with the handle),
+// so feasibility of a split-K launch does not depend on the handle.  `ws_bytes` / `cnt_len` say
+// how much a launch may use; `ws` may still be null while they are non-zero (not yet allocated).
 constexpr size_t kWorkspaceBytes = 64u << 20;
 constexpr int    kCounters       = 1 << 16;
 struct Scratch {
@@ -46,12 +51,40 @@ struct Scratch {
     int    cnt_len;
 };
 
+// Launches `kernel` and returns this launch's own status.  (The triple-chevron form reports through
+// hipGetLastError, which also returns - and clears - an error some earlier call of the caller left behind.)
+template<typename... P, typename... A>
+inline hipError_t launch_kernel(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds, hipStream_t st, A... args)
+{
+    std::tuple<P...> held{static_cast<P>(args)...};
+    void*            ptrs[sizeof...(P) > 0 ? sizeof...(P) : 1];
+    int              i = 0;
+    std::apply([&](auto&... v) { ((ptrs[i++] = (void*)&v), ...); }, held);
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, ptrs, lds, st);
+}
+
+// Raises a kernel's dynamic LDS limit once per kernel instantiation (`done`: one bit per device) and
+// device; kernels that ask for more than 64 KiB need it before their first launch on a device.
+inline hipError_t raise_lds_limit(const void* kernel, int bytes, std::atomic<uint64_t>& done)
+{
+    int        dev = 0;
+    hipError_t e   = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+    return e;
+}
+
 int         algo_count();
 const Algo& algo_at(int id);
-// true if algo `id` can run the shape
-bool algo_feasible(int id, int N, int T, int K);
+// true if algo `id` can run the shape with the scratch `lim` allows
+bool algo_feasible(int id, int N, int T, int K, const Scratch& lim);
+// bytes of partial-tile scratch the launch would use (0: the kernel needs neither workspace nor counters)
+size_t algo_scratch_bytes(int id, int N, int T, int K, const Scratch& lim);
 // heuristic choice (the counterpart of Estimate); -1 if nothing is feasible
-int algo_pick(int N, int T, int K);
+int algo_pick(int N, int T, int K, const Scratch& lim);
 // workgroups the launch would use
 int algo_grid(int id, int N, int T, int K, const Scratch& sc);
 hipError_t algo_launch(int id, const GemmArgs& a, const Scratch& sc, hipStream_t st);
@@ -69,6 +102,7 @@ hipError_t launch_from_reference(uint32_t* dst, const uint32_t* ref, int m, int 
 
 // decode (skinny) kernels
 bool       decode_feasible(const DecodeConfig& cf, int N, int T, int K);
+size_t     decode_scratch_bytes(const DecodeConfig& cf, int N, int T, int K, size_t ws_bytes, int cnt_len);
 int        decode_grid(const DecodeConfig& cf, int N, int T, int K, size_t ws_bytes, int cnt_len);
 hipError_t decode_launch(const DecodeConfig& cf, const GemmArgs& a, float* ws, size_t ws_bytes, int* cnt, int cnt_len,
                          hipStream_t st);
@@ -84,7 +118,8 @@ int        prefill_variants();
 void       prefill_tile(int variant, int& tile_n, int& tile_t);
 // `splits` > 1 divides the quantisation groups among that many workgroups per output tile; the
 // last one to arrive adds the partial tiles (in split order) and runs the epilogue.
-bool       prefill_feasible(int variant, int splits, int N, int T, int K);
+bool       prefill_feasible(int variant, int splits, int N, int T, int K, size_t ws_bytes, int cnt_len);
+size_t     prefill_scratch_bytes(int variant, int splits, int N, int T, int K);
 int        prefill_grid(int variant, int splits, int N, int T, int K);
 hipError_t prefill_launch(int variant, int splits, const GemmArgs& a, const Scratch& sc, hipStream_t st);
 double     prefill_estimate_us(int variant, int splits, int N, int T, int K);  // model fitted to measurements
