@@ -10,7 +10,10 @@
 #include <hip/hip_runtime_api.h>
 
 #include <array>
+#include <iomanip>
+#include <iostream>
 #include <limits>
+#include <ostream>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -26,14 +29,31 @@ struct Metric {
     bool               feasible;
     bool               prefer;
     std::array<int, 3> cta_shape;  // {features, tokens, K slices per workgroup}
-    int                kind;       // 0 decode kernel, 1 MFMA prefill kernel
+    int                kind;       // 0 decode kernel (column blocks), 1 MFMA prefill kernel, 2 decode kernel (strips)
     float              grid_size;
     int                best;
     float              time;       // milliseconds for `count` launches
     int                count;
 };
 
-// gemm_s4_f16.h:15 (kept for source compatibility; nothing is dumped)
+// metric.h:56-110: one line per kernel configuration, in the order given.  The columns are this
+// library's (tile, kernel family, grid, time per launch), not the CUDA occupancy model's.
+inline void DumpMetrics(std::ostream& os, const std::vector<Metric>& metrics)
+{
+    static const char* const kKind[] = {"decode", "mfma", "strip"};
+    os << std::setw(4) << "id" << std::setw(7) << "valid" << std::setw(9) << "kind" << std::setw(10) << "features"
+       << std::setw(8) << "tokens" << std::setw(9) << "k_parts" << std::setw(8) << "grid" << std::setw(12) << "time_us"
+       << std::setw(6) << "best" << "\n";
+    for (const Metric& m : metrics) {
+        os << std::setw(4) << m.id << std::setw(7) << m.feasible << std::setw(9)
+           << (m.kind >= 0 && m.kind <= 2 ? kKind[m.kind] : "?") << std::setw(10) << m.cta_shape[0] << std::setw(8)
+           << m.cta_shape[1] << std::setw(9) << m.cta_shape[2] << std::setw(8) << (int)m.grid_size << std::setw(12)
+           << m.time * 1000 / m.count << std::setw(6) << (m.best ? "*" : "") << "\n";
+    }
+}
+
+// gemm_s4_f16.h:15: when set, the next Measure prints its table to stderr once and clears the flag
+// (gemm_s4_f16.cu:160-163)
 inline bool g_dump_kernel_info_once = false;
 
 class GemmS4F16 {
@@ -126,6 +146,10 @@ public:
             x.time      = r.ms;
             x.count     = r.count;
             metrics.push_back(x);
+        }
+        if (g_dump_kernel_info_once) {
+            DumpMetrics(std::cerr, metrics);
+            g_dump_kernel_info_once = false;
         }
     }
 

@@ -83,9 +83,10 @@ void w4a16_destroy(w4a16_handle* h);
  * for W4A16_FUSED_SILU_FFN).
  * Numerics: the kernels for up to 32 tokens (and narrow matrices up to ~128) scale each group's
  * fp32 partial sum by the fp16 scale; the MFMA prefill kernels multiply by the fp16 weight
- * fp16((q - z) * s), without the reference's flush of subnormal products to zero (common.h:229-230
- * mul.ftz; only w4a16_dequantize_repacked flushes).  Both are within the 1e-2 tolerance of each
- * other and of the reference, but not bit-identical: the same input can give different bits on the
+ * fp16((q - z) * s).  Both treat a subnormal scale as zero, which is all that the reference's
+ * flush-to-zero multiply (common.h:229-230 mul.ftz) ever does: a normal scale times a non-zero
+ * integer is never subnormal.  The two families are within the 1e-2 tolerance of each other and of
+ * the reference, but not bit-identical: the same input can give different bits on the
  * two sides of a hand-over point between kernel families. */
 int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R,
                int n_out, int tokens, int k, int group_size, int epilogue, int algo_id, void* stream);

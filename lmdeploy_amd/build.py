@@ -123,7 +123,7 @@ def check_headers(verbose: bool = True) -> str:
     cmd = [_hipcc(), "-x", "hip", "--offload-arch=gfx950", "-std=c++17", "-O1", "-Wall",
            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
            "-I", os.path.join(root, "include"), src, "-o", out, "-L", LIB_DIR, "-lw4a16",
-           "-Wl,-rpath," + LIB_DIR]
+           "-Wl,-rpath,$ORIGIN/../lib"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("drop-in header check failed:\n%s\n%s" % (r.stdout, r.stderr))

@@ -183,7 +183,7 @@ decode_kernel(const DecodeParams p)
             // Convert the scale now and hide it from the optimiser: otherwise the conversion is
             // folded into the final multiply-add, the Q word stays live past the refill of this
             // stage, and the refill needs a copy that waits for every load in flight.
-            float sf = (float)h[1];
+            float sf = scale_is_normal(s.q[r]) ? (float)h[1] : 0.f;
             asm volatile("" : "+v"(sf));
             float4_t g4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll

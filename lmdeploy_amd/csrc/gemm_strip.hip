@@ -207,7 +207,7 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
                 // Convert the scale now and hide it from the optimiser: otherwise the conversion is
                 // folded into the final multiply-add, the Q word stays live past the refill of this
                 // stage, and the refill lands in a copy that is moved back while still in flight.
-                sf[u] = (float)h2[1];
+                sf[u] = scale_is_normal(s.q[r]) ? (float)h2[1] : 0.f;
                 asm volatile("" : "+v"(sf[u]));
 #pragma unroll
                 for (int h = 0; h < H; ++h) g4[h][u] = float4_t{0.f, 0.f, 0.f, 0.f};

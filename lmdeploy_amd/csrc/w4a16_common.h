@@ -102,6 +102,14 @@ __device__ __forceinline__ half8_t dequant_full(uint32_t w, half2_t z1024, half2
     return r;
 }
 
+// The reference multiplies (q - z) by the scale with flush-to-zero (mul.ftz.f16x2, common.h:229-230):
+// a subnormal scale counts as zero, and that is the only case in which the flush acts, because a
+// normal scale times a non-zero integer is never subnormal.  True if the scale of Q word `q` is normal.
+__device__ __forceinline__ bool scale_is_normal(uint32_t q)
+{
+    return (q & 0x7c000000u) != 0;
+}
+
 // A Q entry is half2(64 + z, s) with bits 0x5400 | z << 4 in the low half.
 __device__ __forceinline__ void split_q(uint32_t q, half2_t& z1024, half2_t& z64, half_t& s)
 {
@@ -109,7 +117,7 @@ __device__ __forceinline__ void split_q(uint32_t q, half2_t& z1024, half2_t& z64
     z64             = half2_t{h[0], h[0]};
     const uint32_t zb = ((q >> 4) & 0xfu) | 0x6400u;
     z1024           = as_half2(zb | (zb << 16));
-    s               = h[1];
+    s               = scale_is_normal(q) ? h[1] : (half_t)0.f;
 }
 
 }  // namespace w4a16

@@ -292,6 +292,15 @@ def max_abs_rel(y: np.ndarray, yref: np.ndarray) -> float:
     return float(np.max(np.abs(y64 - r64))) / (den if den > 0 else 1.0)
 
 
+def elementwise_pass_rate(y: np.ndarray, yref: np.ndarray, rtol: float = 1e-2) -> float:
+    """Share of the outputs with |y - yref| <= rtol * |yref| + rtol * rms(yref): the elementwise
+    reading of the tolerance, which unlike the max-norm gate also holds small outputs to account."""
+    y64, r64 = y.astype(np.float64), yref.astype(np.float64)
+    rms = float(np.sqrt(np.mean(r64 * r64))) if r64.size else 0.0
+    ok = np.abs(y64 - r64) <= rtol * np.abs(r64) + rtol * rms
+    return float(np.mean(ok)) if ok.size else 1.0
+
+
 # ---------------------------------------------------------------------------
 # The gfx950 tiled layout produced by this build's convert_s4_k_m8 (specification).
 # ---------------------------------------------------------------------------

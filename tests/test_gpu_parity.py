@@ -2,7 +2,8 @@
 
 Integer work (repack, unpack, fuse, transpose, dequantised weights) must be bit exact.
 GEMM outputs must satisfy max|y - yref| / max|yref| <= 1e-2 in fp16 (the stated tolerance),
-and are exact in the special cases where the mathematics fixes the answer."""
+and are exact in the special cases where the mathematics fixes the answer.  On the benchmark
+configurations every single output must also satisfy |y - yref| <= 1e-2 |yref| + 1e-2 rms(yref)."""
 import numpy as np
 import pytest
 import torch
@@ -33,6 +34,13 @@ def dev(a: np.ndarray) -> torch.Tensor:
 
 def host_u32(t: torch.Tensor) -> np.ndarray:
     return t.cpu().numpy().view(np.uint32)
+
+
+def assert_close(got, want, what):
+    """The max-norm gate plus the elementwise criterion (pass rate must be 100 %)."""
+    err = O.max_abs_rel(got, want)
+    rate = O.elementwise_pass_rate(got, want, TOL)
+    assert np.isfinite(got).all() and err <= TOL and rate == 1.0, (what, err, rate)
 
 
 def convert(tm, d, N, K):
@@ -236,6 +244,84 @@ def test_residual_in_place(tm, gemm):
     assert O.max_abs_rel(C.cpu().numpy(), want) <= TOL
 
 
+@pytest.fixture(scope="module")
+def algo_table(tm, gemm):
+    """id -> (kind, tokens per workgroup, K parts) of every kernel configuration (they do not depend on the shape)."""
+    T, K, N = 4, 256, 64
+    d = O.make_inputs(1, T, K, N)
+    A, Q = convert(tm, d, N, K)
+    ms = gemm.Measure(torch.empty(T, N, dtype=torch.float16, device="cuda"), A, dev(d["X"]), Q, N, T, K, 128)
+    gemm.clear_tuning()
+    return {m.id: (m.kind, m.tile_t, m.slices) for m in ms}
+
+
+@pytest.mark.parametrize("N", [16384, 32768, 22016, 17600, 12288])
+def test_strip_kernels_on_wide_matrices(tm, gemm, algo_table, N):
+    """Strips of several column tiles (2 to 8 per workgroup, even and uneven deals of the column tiles to
+    256 and 512 workgroups), every strip configuration forced by id, few groups (so that some waves of a
+    workgroup have none), 16- and 32-token variants, every epilogue."""
+    K = 256
+    strips = [i for i, (kind, _, _) in algo_table.items() if kind == 2]
+    assert len(strips) == 4
+    Ts = (1, 8, 16, 20, 32)
+    d = O.make_inputs(4000 + N, max(Ts), K, N, residual=True)
+    A, Q = convert(tm, d, N, K)
+    W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], 128)
+    ran = 0
+    for T in Ts:
+        dd = dict(d, X=d["X"][:T], R=d["R"][:T])
+        acc = O.gemm_acc(dd["X"], W)
+        for kind in (0, 1, 2):
+            want = O.epilogue(acc, kind, dd["R"] if kind == 2 else None)
+            for algo in strips:
+                try:
+                    got = run(tm, gemm, dd, A, Q, T, K, N, kind, algo)
+                except tm.W4A16Error as e:
+                    assert e.code == -2, e       # the 32-token strips do not take 16 tokens or fewer
+                    assert algo_table[algo][1] == 32 and T <= 16, (algo, T)
+                    continue
+                ran += 1
+                assert_close(got, want, (N, T, kind, algo))
+    assert ran >= 3 * (3 * 2 + 2 * 4)
+
+
+@pytest.mark.parametrize("name,K,N,kind", [("qkv", 4096, 12288, 0), ("gate_up", 4096, 22016, 1)])
+def test_llama7b_wide_shapes_at_17_to_32_tokens_take_the_32_token_strips(tm, gemm, algo_table, name, K, N, kind):
+    """qkv (strips of 3 tiles) and gate_up (strips of 3 and 2: 512 workgroups) with 32 token rows per workgroup:
+    what the default dispatch picks at 17 and 24 tokens, and forced by id at 32 (where the dispatch may prefer
+    an MFMA tile)."""
+    d = O.make_inputs(4100 + kind, 32, K, N)
+    A, Q = convert(tm, d, N, K)
+    W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], 128)
+    strip32 = [i for i, (k, tile_t, _) in sorted(algo_table.items()) if (k, tile_t) == (2, 32)]
+    for T in (17, 24, 32):
+        dd = dict(d, X=d["X"][:T])
+        want = O.epilogue(O.gemm_acc(dd["X"], W), kind)
+        k, tile_t, _ = algo_table[gemm.pick(N, T, K)]
+        if T < 32:
+            assert (k, tile_t) == (2, 32), (name, T, k, tile_t)
+        assert_close(run(tm, gemm, dd, A, Q, T, K, N, kind), want, (name, T, "default"))
+        for algo in strip32:
+            assert_close(run(tm, gemm, dd, A, Q, T, K, N, kind, algo), want, (name, T, algo))
+
+
+def test_subnormal_scales_count_as_zero_in_the_gemm(tm, gemm):
+    """The reference multiplies with flush-to-zero (common.h:229-230): a subnormal scale is read as zero, so such a
+    group contributes nothing (a normal scale times a non-zero integer is never subnormal, so nothing else is ever
+    flushed).  The GEMM kernels do the same; without it this case fails the elementwise criterion."""
+    K, N = 512, 256
+    for T in (4, 100):
+        d = O.make_inputs(4200 + T, T, K, N, residual=True)
+        s = d["scales"].copy()
+        s[1, :] = np.float16(2.0 ** -16)       # every product of this group is subnormal (or zero)
+        s[2, ::2] = np.float16(3.0e-5)
+        d["scales"] = s
+        A, Q = convert(tm, d, N, K)
+        for kind in (0, 1, 2):
+            want = O.gemm_s4_f16(d["X"], d["qweight"], d["qzeros"], s, 128, kind, d["R"])
+            assert_close(run(tm, gemm, d, A, Q, T, K, N, kind), want, (T, kind))
+
+
 # ------------------------------------------------------------------ the benchmark configurations
 LLAMA7B = [("qkv", 4096, 12288, 0), ("o", 4096, 4096, 0), ("gate_up", 4096, 22016, 1), ("down", 11008, 4096, 2)]
 SEED = {"qkv": 11, "o": 22, "gate_up": 33, "down": 44}
@@ -250,8 +336,7 @@ def test_llama7b_decode_shapes(tm, gemm, name, K, N, kind):
         dd = dict(d, X=d["X"][:T], R=d["R"][:T])
         want = O.epilogue(O.gemm_acc(dd["X"], W), kind, dd["R"] if kind == 2 else None)
         got = run(tm, gemm, dd, A, Q, T, K, N, kind)
-        err = O.max_abs_rel(got, want)
-        assert err <= TOL, (name, T, err)
+        assert_close(got, want, (name, T))
 
 
 @pytest.mark.parametrize("name,K,N,kind", LLAMA7B)
@@ -266,8 +351,8 @@ def test_llama7b_prefill_shapes_sampled_rows(tm, gemm, name, K, N, kind):
     rows = np.unique(np.concatenate([[0, 1, 15, 16, 255, 256, T - 1], rng.integers(0, T, 89)]))
     W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], 128)
     want = O.epilogue(O.gemm_acc(d["X"][rows], W), kind, d["R"][rows] if kind == 2 else None)
-    err = O.max_abs_rel(got[rows], want)
-    assert np.isfinite(got).all() and err <= TOL, (name, err)
+    assert np.isfinite(got).all()
+    assert_close(got[rows], want, name)
 
 
 LLAMA70B = [("qkv70", 8192, 10240, 0), ("o70", 8192, 8192, 0), ("gate_up70", 8192, 57344, 1), ("down70", 28672, 8192, 2)]
@@ -294,8 +379,8 @@ def test_llama70b_shapes_sampled_columns(tm, gemm, name, K, N, kind):
         rows = np.arange(T) if T <= 16 else np.unique(np.concatenate([[0, 15, 16, T - 1], rng.integers(0, T, 44)]))
         want = O.epilogue(O.gemm_acc(dd["X"][rows], Wc), kind, dd["R"][rows][:, cols] if kind == 2 else None)
         sel = got[rows][:, pairs] if kind == 1 else got[rows][:, cols]
-        err = O.max_abs_rel(sel, want)
-        assert np.isfinite(got).all() and err <= TOL, (name, T, err)
+        assert np.isfinite(got).all()
+        assert_close(sel, want, (name, T))
 
 
 def test_llama7b_32_layer_decode_sequence(tm, gemm):
@@ -349,8 +434,7 @@ def test_llama7b_32_layer_decode_sequence(tm, gemm):
             qw, qz, sc = tm.unpack_repacked(A, Q, N, K, 128)
             W = O.dequant_from_awq(host_u32(qw), host_u32(qz), sc.cpu().numpy(), 128)
             want = O.epilogue(O.gemm_acc(xin, W), kind, res)
-            err = O.max_abs_rel(got, want)
-            assert err <= TOL, (li, K, N, kind, err)
+            assert_close(got, want, (li, K, N, kind))
 
 
 @pytest.mark.parametrize("K,N", [(1024, 3072), (512, 4112), (128, 16), (2048, 2064), (4224, 1024)])
