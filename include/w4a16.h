@@ -91,6 +91,22 @@ void w4a16_destroy(w4a16_handle* h);
 int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R,
                int n_out, int tokens, int k, int group_size, int epilogue, int algo_id, void* stream);
 
+/* w4a16_gemm for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  It takes
+ * no handle (creating one allocates); where w4a16_gemm's split-K kernels use the handle's workspace,
+ * this entry point uses a buffer that is part of the library's code object: 8 MiB of partial tiles
+ * plus 4096 arrival counters, resident on every GPU the library runs on until the process ends.
+ * Arguments, results and error codes are those of w4a16_gemm.  algo_id < 0 picks among the kernels
+ * whose scratch fits that buffer; an explicit algo_id whose partial tiles for this shape do not
+ * fit (n_out * tokens (padded to the tile) * splits * 4 bytes > 8 MiB, or more than 4096 output
+ * tiles) fails with W4A16_ESCRATCH.  It calls no allocating routine; the buffer's device address
+ * is looked up (hipGetSymbolAddress) by the first call on a device or by w4a16_create.  All calls
+ * on one GPU share the one buffer: calls that can overlap on the GPU (different streams, or
+ * different threads) race, so order them on one stream.  The counters are cleared by a small fill
+ * kernel before every launch that uses them. */
+int w4a16_gemm_static(void* C, const void* A, const void* X, const void* Q, const void* R, int n_out, int tokens,
+                      int k, int group_size, int epilogue, int algo_id, void* stream);
+
 /* The int4 branch of LlamaFfnLayer<T>::forward (src/turbomind/models/llama/LlamaFfnLayer.cc:67-116)
  * as one call: gating = SiLU-gated fused gate/up GEMM (kFusedSiluFfn) into `gating_buf`
  * [tokens, inter_size], then ffn_output = gating * W2 (+ residual if `residual` is not null: the add

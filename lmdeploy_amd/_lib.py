@@ -37,6 +37,7 @@ SIGNATURES = {
     "w4a16_create": (c_int, [POINTER(c_void_p)]),
     "w4a16_destroy": (None, [c_void_p]),
     "w4a16_gemm": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_void_p]),
+    "w4a16_gemm_static": (c_int, [c_void_p] * 5 + [c_int] * 6 + [c_void_p]),
     "w4a16_ffn": (c_int, [c_void_p] * 9 + [c_int] * 4 + [c_void_p]),
     "w4a16_measure": (c_int, [c_void_p] * 6 + [c_int] * 5 + [POINTER(Metric), c_int, c_void_p]),
     "w4a16_algo_count": (c_int, []),

@@ -301,6 +301,9 @@ int w4a16_create(w4a16_handle** out)
     if (e == hipSuccess) e = hipMalloc((void**)&h->scratch.cnt, kCounters * sizeof(int));
     if (e == hipSuccess) e = hipMemset(h->scratch.cnt, 0, kCounters * sizeof(int));
     if (e == hipSuccess) e = hipDeviceSynchronize();
+    // a library set-up call on this device: also the moment to look up the static scratch array's address
+    Scratch st{};
+    if (e == hipSuccess) e = static_scratch(&st);
     if (e != hipSuccess) {
         if (h->ev_start) (void)hipEventDestroy(h->ev_start);
         if (h->ev_end) (void)hipEventDestroy(h->ev_end);
@@ -377,6 +380,39 @@ int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const voi
                n_out,        tokens,             k,                  epilogue};
     const hipError_t e = algo_launch(algo_id, g, sc, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "w4a16_gemm launch");
+    return W4A16_OK;
+}
+
+int w4a16_gemm_static(void* C, const void* A, const void* X, const void* Q, const void* R, int n_out, int tokens,
+                      int k, int group_size, int epilogue, int algo_id, void* stream)
+{
+    const int chk = check_gemm_args(C, A, X, Q, R, n_out, tokens, k, group_size, epilogue);
+    if (chk < 0) return chk;
+    if (chk > 0) return W4A16_OK;
+    if (algo_id >= algo_count()) return fail(W4A16_EALGO, "algo_id %d out of range (0..%d)", algo_id, algo_count() - 1);
+    Scratch sc{};
+    if (const hipError_t e = static_scratch(&sc); e != hipSuccess) return hip_fail(e, "w4a16_gemm_static set-up");
+    if (algo_id < 0) algo_id = algo_pick(n_out, tokens, k, sc);
+    if (algo_id < 0) return fail(W4A16_ESHAPE, "no feasible kernel found");
+    if (!algo_feasible(algo_id, n_out, tokens, k, sc)) {
+        // feasible with a handle's (larger) workspace?  Then it is the static buffer that is too small.
+        Scratch big{nullptr, kWorkspaceBytes, nullptr, kCounters};
+        if (algo_feasible(algo_id, n_out, tokens, k, big))
+            return fail(W4A16_ESCRATCH, "algo %d needs %zu bytes of split-K scratch for this shape; the static buffer holds %zu "
+                                        "bytes and %d counters",
+                        algo_id, algo_scratch_bytes(algo_id, n_out, tokens, k, big), sc.ws_bytes, sc.cnt_len);
+        return fail(W4A16_ESHAPE, "no feasible kernel found");
+    }
+    if (int rc = check_prefill_alignment(algo_id, C, R, epilogue)) return rc;
+    const hipStream_t st = (hipStream_t)stream;
+    if (algo_scratch_bytes(algo_id, n_out, tokens, k, sc) > 0) {
+        // every call on this GPU shares the array, whatever an earlier (perhaps aborted) call left in it
+        if (const hipError_t e = clear_counters(sc, st); e != hipSuccess) return hip_fail(e, "w4a16_gemm_static clear");
+    }
+    GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
+               n_out,        tokens,             k,                  epilogue};
+    const hipError_t e = algo_launch(algo_id, g, sc, st);
+    if (e != hipSuccess) return hip_fail(e, "w4a16_gemm_static launch");
     return W4A16_OK;
 }
 

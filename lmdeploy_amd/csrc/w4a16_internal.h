@@ -89,6 +89,14 @@ int algo_pick(int N, int T, int K, const Scratch& lim);
 int algo_grid(int id, int N, int T, int K, const Scratch& sc);
 hipError_t algo_launch(int id, const GemmArgs& a, const Scratch& sc, hipStream_t st);
 
+// The scratch that lives in a file-scope device array (static_scratch.hip), for callers that cannot
+// allocate: its address on the current device, looked up once per device.
+constexpr size_t kStaticCounters       = 4096;
+constexpr size_t kStaticWorkspaceBytes = 8u << 20;
+hipError_t static_scratch(Scratch* out);
+// zeroes the arrival counters of `sc` with a fill kernel on `st`
+hipError_t clear_counters(const Scratch& sc, hipStream_t st);
+
 hipError_t launch_convert(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* A_src, const uint16_t* scales,
                           const uint32_t* qzeros, int m, int k, hipStream_t st);
 hipError_t launch_unpack(uint32_t* qweight, uint32_t* qzeros, uint16_t* scales, const uint32_t* A,

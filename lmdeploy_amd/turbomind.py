@@ -91,6 +91,14 @@ def from_reference_layout(A_ref, m: int, k: int):
     return out
 
 
+def gemm_static(C, A, B, Q, m: int, n: int, k: int, group_size: int, type: int = 0, algo_id: int = -1,
+                residual=None, stream: Optional[int] = None) -> None:
+    """`GemmS4F16.Run` without a handle and without any allocation: split-K kernels use the scratch
+    buffer inside the library (8 MiB per GPU, shared by all calls on that GPU)."""
+    check(lib.w4a16_gemm_static(_ptr(C), _ptr(A), _ptr(B), _ptr(Q), _ptr(residual), m, n, k, group_size, type,
+                                algo_id, _stream() if stream is None else stream))
+
+
 class GemmS4F16:
     """gemm_s4_f16.h:17-56.  `Run(C, A, B, Q, m, n, k, group_size, type, algo_id)` with m = output
     features, n = tokens; B is the fp16 activation matrix [n, k]."""
