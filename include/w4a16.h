@@ -31,6 +31,7 @@ extern "C" {
 #define W4A16_EARG (-4)      /* null pointer / negative size / bad enum      */
 #define W4A16_EALGO (-5)     /* algo_id out of range                         */
 #define W4A16_ESCRATCH (-6)  /* the split-K scratch this launch needs is not available */
+#define W4A16_ETIMEOUT (-7)  /* a device-wide barrier of w4a16_gemm_sequence gave up       */
 
 /* epilogues; 0 and 1 are GemmS4F16::Type (gemm_s4_f16.h:23-27), 2 is an extension */
 #define W4A16_GEMM 0
@@ -107,13 +108,58 @@ int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const voi
 int w4a16_gemm_static(void* C, const void* A, const void* X, const void* Q, const void* R, int n_out, int tokens,
                       int k, int group_size, int epilogue, int algo_id, void* stream);
 
+/* One GEMM of a sequence: the arguments of w4a16_gemm that differ from GEMM to GEMM. */
+typedef struct w4a16_gemm_desc {
+    void*       C;
+    const void* A;
+    const void* X;
+    const void* Q;
+    const void* R;        /* residual for W4A16_FUSED_ADD (may alias C), else NULL                    */
+    int         n_out;
+    int         k;
+    int         epilogue;
+    int         depends;  /* non-zero: this GEMM reads (X or R) what an earlier GEMM of the list writes,
+                             or writes what an earlier one reads or writes; 0: it may overlap with them */
+} w4a16_gemm_desc;
+
+/* A list of GEMMs with a common token count, executed as if by `count` calls of w4a16_gemm (algo_id
+ * -1) in list order, e.g. the four GEMMs of a decoder layer (LlamaDecoder.cc:205-235:
+ * qkv, o - LlamaDecoderSelfAttentionLayer.cc:236-292 -, then LlamaFfnLayer.cc:87-103), or those of
+ * several layers.
+ * flags = 0: one launch per GEMM on `stream`.
+ * flags = W4A16_SEQ_PERSISTENT, up to 16 tokens: the whole list (32 GEMMs at a time) runs as ONE
+ * persistent launch of one workgroup per CU.  A GEMM with `depends` set starts behind a device-wide
+ * barrier (outputs written through at agent scope, arrival on a two-level counter tree, activations
+ * read at agent scope), across which the first weight tiles of the next GEMM are already in flight.
+ * Results are bit-identical to w4a16_gemm with the strip kernel (one strip per CU).  Measured on
+ * MI355X this is SLOWER than one launch per GEMM (a Llama-2-7B layer at 8 tokens: 44 us against 34
+ * us inside a HIP graph): crossing the barrier costs 3 - 4.5 us per GEMM, a launch about 3 us.  It is
+ * kept for callers for whom launches are dearer than that (no graphs, a busy host thread).
+ * The persistent launch needs its workgroups resident all at once, which holds when nothing else
+ * occupies the GPU's CUs for long; its barrier waits are bounded (w4a16_set_barrier_timeout, default
+ * 2 s): a workgroup that gives up sets an error word in the handle, and every workgroup still
+ * finishes.  Nothing is allocated and nothing synchronises, so the call can be captured in a HIP
+ * graph (for T > 16, and for matrices that split K, after one call outside capture: see w4a16_create). */
+#define W4A16_SEQ_PERSISTENT 1
+int w4a16_gemm_sequence(w4a16_handle* h, const w4a16_gemm_desc* gemms, int count, int tokens, int group_size,
+                        int flags, void* stream);
+
+/* Synchronises `stream` and reports whether a barrier of an earlier w4a16_gemm_sequence on this handle
+ * gave up: W4A16_OK, or W4A16_ETIMEOUT (once; the handle is usable again afterwards). */
+int w4a16_sequence_status(w4a16_handle* h, void* stream);
+
+/* Time limit of one barrier wait of w4a16_gemm_sequence, 0 .. 3600 seconds. */
+int w4a16_set_barrier_timeout(w4a16_handle* h, double seconds);
+
 /* The int4 branch of LlamaFfnLayer<T>::forward (src/turbomind/models/llama/LlamaFfnLayer.cc:67-116)
  * as one call: gating = SiLU-gated fused gate/up GEMM (kFusedSiluFfn) into `gating_buf`
  * [tokens, inter_size], then ffn_output = gating * W2 (+ residual if `residual` is not null: the add
  * half of the fused add-norm that follows in LlamaDecoder.cc:228-235; `residual` may alias
  * `ffn_output`).  A13/Q13 are the converted fused w1|w3 weights (n_out = 2 * inter_size, k =
- * hidden_units), A2/Q2 the converted w2 (n_out = hidden_units, k = inter_size).  Both launches go to
- * `stream` back to back; nothing is allocated, so the call can be captured in a HIP graph. */
+ * hidden_units), A2/Q2 the converted w2 (n_out = hidden_units, k = inter_size).  It is the two-GEMM
+ * w4a16_gemm_sequence with flags 0: two launches back to back on `stream` (a single persistent
+ * launch was built and measured slower, see there).  Nothing is allocated, so the call can be
+ * captured in a HIP graph. */
 int w4a16_ffn(w4a16_handle* h, void* ffn_output, void* gating_buf, const void* ffn_input, const void* A13,
               const void* Q13, const void* A2, const void* Q2, const void* residual, int hidden_units,
               int inter_size, int tokens, int group_size, void* stream);

@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_size_t, c_void_p
+from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_size_t, c_void_p
 
 # The callers hand over torch tensors, so torch is in the process anyway - and it must come first:
 # torch ships its own libamdhip64 and libw4a16.so has to bind to that same HIP runtime.  Loaded the
@@ -16,14 +16,21 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # W4A16_LIB overrides the in-tree library (e.g. to try a differently tuned build)
 LIB_PATH = os.environ.get("W4A16_LIB") or os.path.join(_HERE, "lib", "libw4a16.so")
 
-OK, EGROUP, ESHAPE, EHIP, EARG, EALGO, ESCRATCH = 0, -1, -2, -3, -4, -5, -6
+OK, EGROUP, ESHAPE, EHIP, EARG, EALGO, ESCRATCH, ETIMEOUT = 0, -1, -2, -3, -4, -5, -6, -7
 GEMM, FUSED_SILU_FFN, FUSED_ADD = 0, 1, 2
+SEQ_PERSISTENT = 1
 
 
 class Metric(Structure):
     """struct w4a16_metric of include/w4a16.h."""
     _fields_ = [("id", c_int), ("feasible", c_int), ("best", c_int), ("kind", c_int), ("tile_n", c_int),
                 ("tile_t", c_int), ("slices", c_int), ("grid", c_int), ("ms", c_float), ("count", c_int)]
+
+
+class GemmDesc(Structure):
+    """struct w4a16_gemm_desc of include/w4a16.h."""
+    _fields_ = [("C", c_void_p), ("A", c_void_p), ("X", c_void_p), ("Q", c_void_p), ("R", c_void_p),
+                ("n_out", c_int), ("k", c_int), ("epilogue", c_int), ("depends", c_int)]
 
 
 class W4A16Error(RuntimeError):
@@ -38,6 +45,9 @@ SIGNATURES = {
     "w4a16_destroy": (None, [c_void_p]),
     "w4a16_gemm": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_void_p]),
     "w4a16_gemm_static": (c_int, [c_void_p] * 5 + [c_int] * 6 + [c_void_p]),
+    "w4a16_gemm_sequence": (c_int, [c_void_p, POINTER(GemmDesc), c_int, c_int, c_int, c_int, c_void_p]),
+    "w4a16_sequence_status": (c_int, [c_void_p, c_void_p]),
+    "w4a16_set_barrier_timeout": (c_int, [c_void_p, c_double]),
     "w4a16_ffn": (c_int, [c_void_p] * 9 + [c_int] * 4 + [c_void_p]),
     "w4a16_measure": (c_int, [c_void_p] * 6 + [c_int] * 5 + [POINTER(Metric), c_int, c_void_p]),
     "w4a16_algo_count": (c_int, []),

@@ -48,6 +48,10 @@ struct w4a16_handle {
     hipEvent_t     ev_end{};
     int            device{};
     w4a16::Scratch scratch{};
+    int*           sync{};        // counters of the device-wide barrier of w4a16_gemm_sequence
+    int            cus{};         // compute units of the device: workgroups of a persistent launch
+    long long      clock_khz{};   // rate of the device's wall clock
+    long long      spin_ticks{};  // time limit of one barrier wait
     // fastest kernel found by w4a16_measure, per (n_out, tokens, k); consulted before the heuristic
     std::map<std::tuple<int, int, int>, int> tuned;
 };
@@ -300,6 +304,13 @@ int w4a16_create(w4a16_handle** out)
     if (e == hipSuccess) e = hipEventCreate(&h->ev_end);
     if (e == hipSuccess) e = hipMalloc((void**)&h->scratch.cnt, kCounters * sizeof(int));
     if (e == hipSuccess) e = hipMemset(h->scratch.cnt, 0, kCounters * sizeof(int));
+    if (e == hipSuccess) e = hipMalloc((void**)&h->sync, kSyncInts * sizeof(int));
+    if (e == hipSuccess) e = hipMemset(h->sync, 0, kSyncInts * sizeof(int));
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&h->cus, hipDeviceAttributeMultiprocessorCount, h->device);
+    int khz = 0;
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, h->device);
+    h->clock_khz  = khz > 0 ? khz : 100000;
+    h->spin_ticks = 2000 * h->clock_khz;  // two seconds
     if (e == hipSuccess) e = hipDeviceSynchronize();
     // a library set-up call on this device: also the moment to look up the static scratch array's address
     Scratch st{};
@@ -308,6 +319,7 @@ int w4a16_create(w4a16_handle** out)
         if (h->ev_start) (void)hipEventDestroy(h->ev_start);
         if (h->ev_end) (void)hipEventDestroy(h->ev_end);
         if (h->scratch.cnt) (void)hipFree(h->scratch.cnt);
+        if (h->sync) (void)hipFree(h->sync);
         delete h;
         return hip_fail(e, "w4a16_create");
     }
@@ -325,6 +337,7 @@ void w4a16_destroy(w4a16_handle* h)
     (void)hipEventDestroy(h->ev_start);
     if (h->scratch.ws) (void)hipFree(h->scratch.ws);
     (void)hipFree(h->scratch.cnt);
+    (void)hipFree(h->sync);
     delete h;
 }
 
@@ -416,16 +429,76 @@ int w4a16_gemm_static(void* C, const void* A, const void* X, const void* Q, cons
     return W4A16_OK;
 }
 
+int w4a16_gemm_sequence(w4a16_handle* h, const w4a16_gemm_desc* gemms, int count, int tokens, int group_size,
+                        int flags, void* stream)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    if (count < 0 || (count > 0 && !gemms)) return fail(W4A16_EARG, "bad sequence");
+    if (flags & ~W4A16_SEQ_PERSISTENT) return fail(W4A16_EARG, "unknown sequence flags %d", flags);
+    // validate everything before anything is launched
+    for (int i = 0; i < count; ++i) {
+        const w4a16_gemm_desc& d = gemms[i];
+        const int chk = check_gemm_args(d.C, d.A, d.X, d.Q, d.R, d.n_out, tokens, d.k, group_size, d.epilogue);
+        if (chk < 0) return chk;
+        if (chk > 0 && tokens != 0) return fail(W4A16_EARG, "GEMM %d of the sequence is empty", i);
+    }
+    if (tokens == 0 || count == 0) return W4A16_OK;
+    if (!(flags & W4A16_SEQ_PERSISTENT) || tokens > 16 || count == 1) {
+        // one launch per GEMM; stream order gives the dependencies
+        for (int i = 0; i < count; ++i) {
+            const w4a16_gemm_desc& d = gemms[i];
+            const int rc = w4a16_gemm(h, d.C, d.A, d.X, d.Q, d.R, d.n_out, tokens, d.k, group_size, d.epilogue, -1, stream);
+            if (rc != W4A16_OK) return rc;
+        }
+        return W4A16_OK;
+    }
+    SeqGemm chunk[kSeqMax];
+    for (int first = 0; first < count; first += kSeqMax) {
+        const int n = std::min(kSeqMax, count - first);
+        for (int i = 0; i < n; ++i) {
+            const w4a16_gemm_desc& d = gemms[first + i];
+            chunk[i] = SeqGemm{(uint16_t*)d.C, (const u32x4_t*)d.A, (const uint16_t*)d.X, (const uint32_t*)d.Q,
+                               (const uint16_t*)d.R, d.n_out, d.k, d.epilogue, (i > 0 && d.depends) ? 1 : 0};
+        }
+        if (!sequence_feasible(chunk, n, tokens)) return fail(W4A16_ESHAPE, "no feasible kernel found");
+        const hipError_t e = sequence_launch(chunk, n, tokens, h->sync, h->cus, h->spin_ticks, (hipStream_t)stream);
+        if (e != hipSuccess) return hip_fail(e, "w4a16_gemm_sequence launch");
+    }
+    return W4A16_OK;
+}
+
+int w4a16_sequence_status(w4a16_handle* h, void* stream)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    hipError_t e = hipStreamSynchronize((hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "w4a16_sequence_status");
+    int word = 0;
+    e = hipMemcpy(&word, h->sync + sequence_error_index(), sizeof(int), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return hip_fail(e, "w4a16_sequence_status");
+    if (word == 0) return W4A16_OK;
+    e = hipMemset(h->sync, 0, kSyncInts * sizeof(int));  // the launch that gave up may have left counters behind
+    if (e != hipSuccess) return hip_fail(e, "w4a16_sequence_status");
+    return fail(W4A16_ETIMEOUT, "a workgroup of w4a16_gemm_sequence gave up waiting at a device-wide barrier: the "
+                                "grid was not resident all at once; the outputs of that launch are undefined");
+}
+
+int w4a16_set_barrier_timeout(w4a16_handle* h, double seconds)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    if (!(seconds >= 0.0) || seconds > 3600.0) return fail(W4A16_EARG, "timeout out of range");
+    h->spin_ticks = (long long)(seconds * 1000.0 * (double)h->clock_khz);
+    return W4A16_OK;
+}
+
 int w4a16_ffn(w4a16_handle* h, void* ffn_output, void* gating_buf, const void* ffn_input, const void* A13,
               const void* Q13, const void* A2, const void* Q2, const void* residual, int hidden_units,
               int inter_size, int tokens, int group_size, void* stream)
 {
     if (hidden_units < 0 || inter_size < 0) return fail(W4A16_EARG, "negative size");
-    const int rc = w4a16_gemm(h, gating_buf, A13, ffn_input, Q13, nullptr, 2 * inter_size, tokens, hidden_units,
-                              group_size, W4A16_FUSED_SILU_FFN, -1, stream);
-    if (rc != W4A16_OK) return rc;
-    return w4a16_gemm(h, ffn_output, A2, gating_buf, Q2, residual, hidden_units, tokens, inter_size, group_size,
-                      residual ? W4A16_FUSED_ADD : W4A16_GEMM, -1, stream);
+    const w4a16_gemm_desc seq[2] = {
+        {gating_buf, A13, ffn_input, Q13, nullptr, 2 * inter_size, hidden_units, W4A16_FUSED_SILU_FFN, 0},
+        {ffn_output, A2, gating_buf, Q2, residual, hidden_units, inter_size, residual ? W4A16_FUSED_ADD : W4A16_GEMM, 1}};
+    return w4a16_gemm_sequence(h, seq, 2, tokens, group_size, 0, stream);
 }
 
 int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R, int n_out,

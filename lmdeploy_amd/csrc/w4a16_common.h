@@ -5,13 +5,14 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "w4a16_internal.h"
+
 namespace w4a16 {
 
 typedef _Float16 half_t;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef float    float4_t __attribute__((ext_vector_type(4)));
 typedef float    float16_t __attribute__((ext_vector_type(16)));
 

@@ -9,6 +9,8 @@
 
 namespace w4a16 {
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
 enum Epilogue { kEpiGemm = 0, kEpiSilu = 1, kEpiAdd = 2 };
 
 struct GemmArgs {
@@ -120,6 +122,24 @@ bool       strip_feasible(int per_cu, int block_t, int N, int T, int K);
 int        strip_grid(int per_cu, int block_t, int N, int T, int K);
 int        strip_width(int per_cu, int block_t, int N, int T, int K);  // column tiles of the widest strip
 hipError_t strip_launch(int per_cu, int block_t, const GemmArgs& a, hipStream_t st);
+
+// A sequence of decode GEMMs (up to 16 tokens) in one persistent launch (gemm_sequence.hip)
+struct SeqGemm {
+    uint16_t*       C;
+    const u32x4_t*  A;
+    const uint16_t* X;
+    const uint32_t* Q;
+    const uint16_t* R;
+    int             N, K;
+    int             epilogue;
+    int             flags;  // bit 0: reads what an earlier GEMM of the sequence writes - wait for all of them
+};
+constexpr int kSeqMax   = 32;    // GEMMs per launch (the descriptors travel as kernel arguments)
+constexpr int kSyncInts = 64 * 80;  // arrival counters, flag, error word of the device-wide barrier
+bool       sequence_feasible(const SeqGemm* g, int count, int T);
+int        sequence_error_index();  // index of the error word in the sync area
+// `cus` workgroups (one per CU: they must all be resident at once); `spin_ticks` bounds each barrier wait
+hipError_t sequence_launch(const SeqGemm* g, int count, int T, int* sync, int cus, long long spin_ticks, hipStream_t st);
 
 // MFMA prefill kernels
 int        prefill_variants();

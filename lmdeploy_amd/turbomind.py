@@ -16,7 +16,7 @@ from typing import List, Optional
 import torch
 
 from . import _lib
-from ._lib import Metric, W4A16Error, check, lib  # noqa: F401
+from ._lib import GemmDesc, Metric, W4A16Error, check, lib  # noqa: F401
 
 
 def _stream() -> int:
@@ -141,6 +141,27 @@ class GemmS4F16:
         check(lib.w4a16_ffn(self._h, _ptr(ffn_output), _ptr(gating_buf), _ptr(ffn_input), _ptr(A13), _ptr(Q13),
                             _ptr(A2), _ptr(Q2), _ptr(residual), hidden_units, inter_size, n, group_size,
                             _stream() if stream is None else stream))
+
+    def sequence(self, gemms, n: int, group_size: int = 128, persistent: bool = False, stream: Optional[int] = None):
+        """A list of GEMMs with a common token count `n` in one call.  `gemms`: tuples
+        (C, A, B, Q, m, k, type, residual, depends) in execution order; `depends` says that the GEMM reads
+        what an earlier one of the list writes.  `persistent`: up to 16 tokens, one persistent launch for the
+        whole list instead of one launch per GEMM.  Returns the descriptor array (the tensors must stay
+        alive while a captured call is replayed)."""
+        arr = (GemmDesc * len(gemms))()
+        for d, (C, A, B, Q, m, k, type_, residual, depends) in zip(arr, gemms):
+            d.C, d.A, d.X, d.Q, d.R = _ptr(C), _ptr(A), _ptr(B), _ptr(Q), _ptr(residual)
+            d.n_out, d.k, d.epilogue, d.depends = m, k, type_, int(bool(depends))
+        check(lib.w4a16_gemm_sequence(self._h, arr, len(gemms), n, group_size,
+                                      _lib.SEQ_PERSISTENT if persistent else 0, _stream() if stream is None else stream))
+        return arr
+
+    def sequence_status(self, stream: Optional[int] = None) -> None:
+        """Synchronises and raises W4A16Error (code -7) if a barrier of an earlier `sequence` gave up."""
+        check(lib.w4a16_sequence_status(self._h, _stream() if stream is None else stream))
+
+    def set_barrier_timeout(self, seconds: float) -> None:
+        check(lib.w4a16_set_barrier_timeout(self._h, seconds))
 
     def pick(self, m: int, n: int, k: int) -> int:
         """The algo_id that `Run(..., algo_id=-1)` uses for this shape: the fastest one a previous
