@@ -2,15 +2,19 @@
 """Benchmark of the W4A16 GEMM path on one MI355X.
 
 A "step" is one pass over the Llama-2-7B decode layer set: the four layer GEMMs
-(qkv, o, gate_up + SiLU, down + residual) at each of T = 1, 4, 8, 16 tokens = 16 launches,
-on a layer copy that differs from step to step (24 copies, about 2.5 GB of packed weights,
-so neither the L2s nor the 256 MB Infinity Cache can serve the weights).  The headline value
-is the aggregate achieved bandwidth: algorithmic bytes of all launches / elapsed time.
+(qkv, o, gate_up + SiLU, down + residual) at each of T = 1, 4, 8, 16 tokens = 16 launches.
+Every one of the 16 GEMMs of a step has its own copy of its weight matrix, and the steps rotate
+through 12 such sets (48 copies per shape, about 5 GB of packed weights), so that no matrix is
+read again before several GB of other traffic have passed: neither the L2s nor the 256 MB
+Infinity Cache can serve the weights.  The headline value is the aggregate achieved bandwidth:
+algorithmic bytes of all launches / elapsed time.
 
-Also reported in the same JSON line: the roofline of the dominant decode kernel (gate_up),
-the prefill (T = 2048) TFLOP/s of the same four shapes with the roofline of its dominant
-kernel, and the CPU baseline (the oracle: unpack, dequantise, torch fp32 matmul) timed on the
-host cores on a bounded sample.
+Also in the same JSON line: roofline objects for the dominant decode kernel (gate_up) and for the
+one furthest below its roofline (o), per-shape tables for Llama-2-7B and Llama-2-70B (decode:
+GB/s; T = 2048: TFLOP/s), the 32-layer decode step at M = 8 as one launch per GEMM and as
+persistent launches, what plain library kernels reach on this GPU (streaming reads of 8 / 45 /
+512 MiB, a device copy, a dense fp16 GEMM), and the CPU baseline (the oracle: unpack,
+dequantise, torch fp32 matmul) timed on the host cores on bounded samples.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 """
@@ -37,7 +41,9 @@ TRAFFIC_PREFILL_GATE_UP = 565.2e6
 
 # name, K, N (gate_up: both halves), epilogue
 LAYER_7B = [("qkv", 4096, 12288, 0), ("o", 4096, 4096, 0), ("gate_up", 4096, 22016, 1), ("down", 11008, 4096, 2)]
+LAYER_70B = [("qkv", 8192, 10240, 0), ("o", 8192, 8192, 0), ("gate_up", 8192, 57344, 1), ("down", 28672, 8192, 2)]
 DECODE_T = (1, 4, 8, 16)
+DECODE_T_70B = (1, 16)
 PREFILL_T = 2048
 BATCHED_T = (32, 64, 128, 256)   # reported per shape, outside the headline metric
 GROUP = 128
@@ -78,17 +84,19 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=96)
     ap.add_argument("--warmup", type=int, default=24)
-    ap.add_argument("--copies", type=int, default=24, help="distinct layer copies the steps rotate through")
+    ap.add_argument("--copies", type=int, default=12,
+                    help="distinct sets of 16 weight matrices (one per GEMM of a step) the steps rotate through")
     ap.add_argument("--cold-gib", type=float, default=1.25,
                     help="per-shape measurements rotate through at least this many GiB of weight copies")
     ap.add_argument("--eager", action="store_true", help="launch from the host instead of replaying HIP graphs")
     ap.add_argument("--prefill-steps", type=int, default=10)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-per-shape", action="store_true")
-    ap.add_argument("--probe", choices=["decode", "prefill"],
-                    help="run only the dominant kernel of that regime plus a plain 256 MiB device copy, "
-                         "eagerly, for `rocprofv3 --pmc` (no JSON line)")
+    ap.add_argument("--no-70b", action="store_true")
+    ap.add_argument("--probe", choices=["decode", "prefill", "decode-o"],
+                    help="run only the named kernel (gate_up decode / gate_up at T=2048 / o decode) plus a plain 256 MiB "
+                         "elementwise kernel, eagerly, for `rocprofv3 --pmc` (no JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -106,16 +114,22 @@ def main():
     gemm = tm.GemmS4F16()
     stream = torch.cuda.Stream()          # default priority; graphs are captured and replayed on it
     shape = {name: (K, N, epi) for name, K, N, epi in LAYER_7B}
+    n_sets = args.copies
     weights = {}
     for name, K, N, epi in LAYER_7B:
         per_copy = K * N // 2 + (K // GROUP) * N * 4
-        n = max(args.copies, N_LAYERS, int(args.cold_gib * 2 ** 30 / per_copy) + 1)
+        n = max(len(DECODE_T) * n_sets, N_LAYERS, int(args.cold_gib * 2 ** 30 / per_copy) + 1)
+        if args.probe:
+            n = max(8, int(args.cold_gib * 2 ** 30 / per_copy) + 1) if name in ("gate_up", "o") else 1
         weights[name] = [make_weights(tm, torch, gen, name, K, N) for _ in range(n)]
     Tmax = max(max(DECODE_T), PREFILL_T)
     X = {K: torch.randn((Tmax, K), device="cuda", generator=gen).half() for K in (4096, 11008)}
     Res = torch.randn((Tmax, 4096), device="cuda", generator=gen).half()
     out = {name: torch.empty((Tmax, N // 2 if epi == 1 else N), dtype=torch.float16, device="cuda")
            for name, K, N, epi in LAYER_7B}
+    # the kernels that split K need the handle's workspace, which cannot be allocated during graph capture
+    gemm.Run(out["down"], *weights["down"][0][:1], X[11008], weights["down"][0][1], 4096, 64, 11008, GROUP, 2, -1,
+             residual=Res)
     torch.cuda.synchronize()
 
     def launch(name, copy, T, st):
@@ -123,18 +137,17 @@ def main():
         A, Q = weights[name][copy % len(weights[name])]
         gemm.Run(out[name], A, X[K], Q, N, T, K, GROUP, epi, -1, residual=Res if epi == 2 else None, stream=st)
 
-    def make_runner(work):
+    def make_runner(work, fn=None):
         """work: list of launch lists; returns one callable per entry (a replayable HIP graph)."""
+        fn = fn or (lambda w, st: [launch(n, c, T, st) for n, c, T in w])
         if args.eager:
-            return [lambda w=w: [launch(n, c, T, stream.cuda_stream) for n, c, T in w] for w in work]
+            return [lambda w=w: fn(w, stream.cuda_stream) for w in work]
         runners = []
         for w in work:
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=stream):
-                st = torch.cuda.current_stream().cuda_stream
-                for n, c, T in w:
-                    launch(n, c, T, st)
-            runners.append(g.replay)
+                keep = fn(w, torch.cuda.current_stream().cuda_stream)
+            runners.append(lambda g=g, keep=keep: g.replay())
         return runners
 
     def timed(runner, steps, warmup):
@@ -151,24 +164,25 @@ def main():
         return e0.elapsed_time(e1)   # ms
 
     if args.probe:
-        # a plain copy of known size calibrates FETCH_SIZE / WRITE_SIZE, then the kernel on cold weights
+        # a plain elementwise kernel of known size calibrates FETCH_SIZE / WRITE_SIZE, then the kernel on cold weights
         src = torch.zeros(64 * 2 ** 20, dtype=torch.int32, device="cuda")   # 256 MiB
         dst = torch.empty_like(src)
+        name = "o" if args.probe == "decode-o" else "gate_up"
         with torch.cuda.stream(stream):
             for _ in range(4):
-                torch.add(src, 1, out=dst)   # an elementwise kernel: reads 256 MiB, writes 256 MiB
-            n = len(weights["gate_up"])
+                torch.add(src, 1, out=dst)   # reads 256 MiB, writes 256 MiB
+            n = len(weights[name])
             for rep in range(2):
                 for c in range(n):
-                    launch("gate_up", c, DECODE_T[c % len(DECODE_T)] if args.probe == "decode" else PREFILL_T,
-                           stream.cuda_stream)
+                    launch(name, c, PREFILL_T if args.probe == "prefill" else DECODE_T[c % len(DECODE_T)], stream.cuda_stream)
         torch.cuda.synchronize()
-        print("probe done: 4 add kernels over 268435456 bytes, %d gate_up launches (%s)" % (2 * n, args.probe))
+        print("probe done: 4 add kernels over 268435456 bytes, %d %s launches (%s)" % (2 * n, name, args.probe))
         return
 
-    # ---- headline: the decode layer set, one layer copy per step ------------------------------
+    # ---- headline: the decode layer set; every GEMM of a step has its own weight copy ----------
     step_bytes = sum(algorithmic_bytes(T, K, N, epi) for T in DECODE_T for _, K, N, epi in LAYER_7B)
-    runner = make_runner([[(name, c, T) for T in DECODE_T for name, _, _, _ in LAYER_7B] for c in range(args.copies)])
+    runner = make_runner([[(name, len(DECODE_T) * c + ti, T) for ti, T in enumerate(DECODE_T) for name, _, _, _ in LAYER_7B]
+                          for c in range(n_sets)])
     ms = timed(runner, args.steps, args.warmup)
     ms_per_step = ms / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
@@ -179,15 +193,19 @@ def main():
         r = make_runner([[(name, c, tokens[c % len(tokens)]) for c in range(n)]])
         return timed(r, passes, 1) * 1e3 / (passes * n)
 
-    # ---- roofline of the dominant decode kernel: gate_up alone, over >= cold-gib of copies -----
-    K, N, _ = shape["gate_up"]
-    gu_bytes = sum(algorithmic_bytes(T, K, N, 1) for T in DECODE_T) / len(DECODE_T)
-    gu_us = per_launch_us("gate_up", DECODE_T, passes=6)
-    achieved = gu_bytes / (gu_us * 1e-6) / 1e9
-    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_DECODE_GATE_UP,
-                "kernel": "strip_kernel, gate_up K=4096 N=22016 +SiLU, T cycling over {1,4,8,16}",
-                "bytes_per_launch": int(gu_bytes), "us_per_launch": round(gu_us, 3)}
+    def decode_roofline(name, traffic, what):
+        K, N, epi = shape[name]
+        by = sum(algorithmic_bytes(T, K, N, epi) for T in DECODE_T) / len(DECODE_T)
+        us = per_launch_us(name, DECODE_T, passes=6)
+        ach = by / (us * 1e-6) / 1e9
+        return {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": what,
+                "bytes_per_launch": int(by), "us_per_launch": round(us, 3)}
+
+    # ---- rooflines: the dominant decode kernel (gate_up) and the one furthest below its roofline (o) ----
+    roofline = decode_roofline("gate_up", TRAFFIC_DECODE_GATE_UP,
+                               "strip_kernel, gate_up K=4096 N=22016 +SiLU, T cycling over {1,4,8,16}")
+    roofline_worst = decode_roofline("o", None, "strip_kernel, o K=4096 N=4096, T cycling over {1,4,8,16}")
 
     # ---- per-shape decode table ----------------------------------------------------------------
     per_shape = []
@@ -230,11 +248,51 @@ def main():
                                 "traffic": TRAFFIC_PREFILL_GATE_UP if dom["shape"] == "gate_up" else None,
                                 "kernel": "prefill_kernel, %s, T=2048" % dom["shape"]}}
 
-    # ---- what this machine reaches with library kernels (context for the two peaks) ------------
-    # a device copy (read + write) for HBM, and hipBLASLt's fp16 GEMM on dense fp16 weights of the
-    # gate_up shape at T = 2048 (what the reference's non-quantised LlamaLinear path would call)
+    # ---- the full 32-layer GEMM sequence of one decode step at M = 8 (every layer its own weights) ----
+    # as one launch per GEMM, and through w4a16_gemm_sequence as persistent launches (32 GEMMs each, every GEMM
+    # behind a device-wide barrier as if it read its predecessor's output)
+    seq_T = 8
+    seq_bytes = N_LAYERS * sum(algorithmic_bytes(seq_T, K, N, epi) for _, K, N, epi in LAYER_7B)
+
+    def layers32(ms_, launch_kind):
+        return {"launch": launch_kind, "ms_per_decode_step": round(ms_, 4), "GBps": round(seq_bytes / ms_ / 1e6, 1),
+                "frac": round(seq_bytes / ms_ / 1e6 / HBM_PEAK_GBS, 4)}
+
+    seq_work = [[(name, layer, seq_T) for layer in range(N_LAYERS) for name, _, _, _ in LAYER_7B]]
+    seq_ms = timed(make_runner(seq_work), 20, 5) / 20
+
+    def persistent(w, st):
+        descs = []
+        for i, (name, c, T) in enumerate(w):
+            K, N, epi = shape[name]
+            A, Q = weights[name][c % len(weights[name])]
+            descs.append((out[name], A, X[K], Q, N, K, epi, Res if epi == 2 else None, i > 0))
+        return gemm.sequence(descs, seq_T, persistent=True, stream=st)
+
+    pers_ms = timed(make_runner(seq_work, persistent), 20, 5) / 20
+    gemm.sequence_status(stream.cuda_stream)
+    layers32_m8 = dict(layers32(seq_ms, "one launch per GEMM (128 launches, one HIP graph)"), T=seq_T, layers=N_LAYERS,
+                       gemms=4 * N_LAYERS,
+                       weights_GB=round(N_LAYERS * sum(K * N // 2 + K // GROUP * N * 4 for _, K, N, _ in LAYER_7B) / 1e9, 2),
+                       persistent=layers32(pers_ms, "w4a16_gemm_sequence, persistent: 4 launches of 32 dependent GEMMs"))
+
+    # ---- what this machine reaches with plain kernels (context for the two peaks) ---------------
+    # a streaming read launched like the decode kernels on 8 / 45 / 512 MiB (cold: rotating through >= 1.25 GiB),
+    # a device copy (read + write), and hipBLASLt's fp16 GEMM on dense fp16 weights of the gate_up shape at
+    # T = 2048 (what the reference's non-quantised LlamaLinear path would call)
     ceilings = None
     if not args.no_prefill:
+        reads = {}
+        for mib in (8, 45, 512):
+            n = max(3, int(args.cold_gib * 1024 / mib) + 1)
+            bufs = [torch.empty(mib << 20, dtype=torch.uint8, device="cuda") for _ in range(n)]
+            for b in bufs:
+                b.zero_()
+            r = make_runner([bufs], lambda w, st: [gemm.probe_read(b, stream=st) for b in w])
+            us = timed(r, 3, 1) * 1e3 / (3 * n)
+            reads["read_%dMiB" % mib] = {"us": round(us, 2), "GBps": round((mib << 20) / us / 1e3, 1),
+                                         "frac": round((mib << 20) / us / 1e3 / HBM_PEAK_GBS, 3)}
+            del bufs, r
         with torch.cuda.stream(stream):
             src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
             dst = torch.empty_like(src)
@@ -260,14 +318,48 @@ def main():
             torch.cuda.synchronize()
             dense_tf = 12 * flops(PREFILL_T, K, N) / e0.elapsed_time(e1) / 1e9
             del Wd, Y
-        ceilings = {"device_copy_512MiB_GBps": round(copy_gbs, 1),
-                    "dense_fp16_gemm_gate_up_T2048_TFLOPs": round(dense_tf, 1),
-                    "note": "torch copy_ (bytes read + written) and torch.matmul fp16 (hipBLASLt) on this GPU"}
+        ceilings = dict(reads, device_copy_512MiB_GBps=round(copy_gbs, 1),
+                        dense_fp16_gemm_gate_up_T2048_TFLOPs=round(dense_tf, 1),
+                        note="read_*: w4a16_probe_read (plain streaming read, one launch per buffer in a HIP graph, cold buffers); "
+                             "torch copy_ (bytes read + written); torch.matmul fp16 (hipBLASLt)")
 
-    # ---- CPU baseline: the oracle on the host cores, one layer at T = 8 -------------------------
+    # ---- Llama-2-70B layer shapes (BASELINE configs[3]) -----------------------------------------
+    llama70b = None
+    if not args.no_70b:
+        rows70 = []
+        X70 = {K: torch.randn((PREFILL_T, K), device="cuda", generator=gen).half() for K in (8192, 28672)}
+        Res70 = torch.randn((PREFILL_T, 8192), device="cuda", generator=gen).half()
+        copies_used = {}
+        for name, K, N, epi in LAYER_70B:
+            per_copy = K * N // 2 + (K // GROUP) * N * 4
+            n = max(3, int(args.cold_gib * 2 ** 30 / per_copy) + 1)
+            copies_used[name] = n
+            ws = [make_weights(tm, torch, gen, name, K, N) for _ in range(n)]
+            C = torch.empty((PREFILL_T, N // 2 if epi == 1 else N), dtype=torch.float16, device="cuda")
+
+            def run70(w, st, K=K, N=N, epi=epi, C=C):
+                for c, T in w:
+                    gemm.Run(C, ws[c][0], X70[K], ws[c][1], N, T, K, GROUP, epi, -1, residual=Res70 if epi == 2 else None,
+                             stream=st)
+            for T in DECODE_T_70B:
+                us = timed(make_runner([[(c, T) for c in range(n)]], run70), 3, 1) * 1e3 / (3 * n)
+                by = algorithmic_bytes(T, K, N, epi)
+                rows70.append({"shape": name, "T": T, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
+                               "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 3)})
+            us = timed(make_runner([[(c, PREFILL_T) for c in range(n)]], run70), 2, 1) * 1e3 / (2 * n)
+            fl = flops(PREFILL_T, K, N)
+            rows70.append({"shape": name, "T": PREFILL_T, "us": round(us, 1), "TFLOPs": round(fl / us / 1e6, 1),
+                           "frac": round(fl / us / 1e6 / MFMA_PEAK_TFLOPS, 4)})
+            del ws, C
+            torch.cuda.empty_cache()
+        llama70b = {"per_shape": rows70, "weight_copies_rotated": copies_used,
+                    "note": "decode rows: frac of 8 TB/s; T=2048 rows: frac of 2.5 PFLOP/s; every launch reads a weight copy "
+                            "that was last touched >= %.2f GiB of traffic ago" % args.cold_gib}
+
+    # ---- CPU baselines: the oracle on the host cores ---------------------------------------------
     cpu = None
+    cpu_prefill = None
     if not args.no_cpu:
-        import numpy as np
         from oracle import w4a16_oracle as O
         T, reps = 8, 5
         t_deq = t_mm = t_mm1 = 0.0
@@ -292,21 +384,26 @@ def main():
             O.epilogue(O.gemm_acc(d["X"], W), epi, d.get("R"))
             t_mm1 += time.perf_counter() - t1
             torch.set_num_threads(nthreads)
+            if name == "o" and not args.no_prefill:
+                # beside the T = 2048 figure: the same path on the o shape (68.7 GFLOP), dequantised weights reused
+                dp = O.make_inputs(99, PREFILL_T, K, N, GROUP)
+                tp = []
+                for _ in range(3):
+                    t1 = time.perf_counter()
+                    O.epilogue(O.gemm_acc(dp["X"], W), epi)
+                    tp.append(time.perf_counter() - t1)
+                tpm = sorted(tp)[1]
+                cpu_prefill = {"value": round(flops(PREFILL_T, K, N) / tpm / 1e12, 4), "unit": "TFLOP/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": "o shape (K=4096, N=4096) at T=2048, torch fp32 matmul + epilogue on already dequantised "
+                                         "weights, median of 3: %.3f s; unpack+dequantise of the matrix adds %.2f s (numpy, 1 thread)"
+                                         % (tpm, sorted(deq)[reps // 2])}
         cpu = {"value": round(by / (t_deq + t_mm) / 1e9, 4), "unit": "GB/s", "cores": torch.get_num_threads(),
                "kind": "port", "host_cpus": os.cpu_count(),
                "sample": "one Llama-2-7B layer (qkv, o, gate_up+SiLU, down+residual) at T=8, median of %d passes per "
                          "GEMM: numpy unpack+dequantise %.2f s (1 thread) + torch fp32 matmul+epilogue %.3f s "
-                         "(%d threads; %.3f s on 1 thread)" % (reps, t_deq, t_mm, torch.get_num_threads(), t_mm1)}
-
-    # ---- the full 32-layer GEMM sequence of one decode step at M = 8 (every layer its own weights) ----
-    seq_T = 8
-    seq_work = [[(name, layer, seq_T) for layer in range(N_LAYERS) for name, _, _, _ in LAYER_7B]]
-    seq_run = make_runner(seq_work)
-    seq_ms = timed(seq_run, 20, 5) / 20
-    seq_bytes = N_LAYERS * sum(algorithmic_bytes(seq_T, K, N, epi) for _, K, N, epi in LAYER_7B)
-    layers32 = {"T": seq_T, "layers": N_LAYERS, "gemms": 4 * N_LAYERS, "ms_per_decode_step": round(seq_ms, 4),
-                "GBps": round(seq_bytes / seq_ms / 1e6, 1), "frac": round(seq_bytes / seq_ms / 1e6 / HBM_PEAK_GBS, 4),
-                "weights_GB": round(N_LAYERS * sum(K * N // 2 + K // GROUP * N * 4 for _, K, N, _ in LAYER_7B) / 1e9, 2)}
+                         "(%d threads; %.3f s on 1 thread)" % (reps, t_deq, t_mm, torch.get_num_threads(), t_mm1),
+               "prefill": cpu_prefill}
 
     line = {
         "metric": "W4A16 GEMM achieved HBM GB/s (M=1..16) + TFLOP/s (M=2048), % of roofline",
@@ -314,14 +411,15 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "Llama-2-7B decode layer set (qkv 4096x12288, o 4096x4096, gate_up 4096x22016 +SiLU, "
-                               "down 11008x4096 +residual) at T in {1,4,8,16}, group 128: 16 GEMMs per step, "
-                               "%d rotating layer copies" % args.copies,
+                               "down 11008x4096 +residual) at T in {1,4,8,16}, group 128: 16 GEMMs per step, each on its own "
+                               "weight copy, %d rotating sets of 16" % n_sets,
                    "launch": "eager" if args.eager else "hipgraph replay of one step",
                    "bytes_per_step": step_bytes},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-        "roofline": roofline, "cpu_baseline": cpu, "decode_per_shape": per_shape, "batched_decode_per_shape": batched,
-        "prefill": prefill,
-        "layers32_m8": layers32, "library_ceilings": ceilings,
+        "roofline": roofline, "roofline_worst_decode_kernel": roofline_worst, "cpu_baseline": cpu,
+        "decode_per_shape": per_shape, "batched_decode_per_shape": batched,
+        "prefill": prefill, "llama70b": llama70b,
+        "layers32_m8": layers32_m8, "library_ceilings": ceilings,
     }
     print(json.dumps(line))
 

@@ -232,6 +232,11 @@ int w4a16_dequantize_repacked(void* W, const uint32_t* A, const void* Q, int m, 
  * layout.  Q needs no conversion.  m % 32 == 0, k % 128 == 0. */
 int w4a16_from_reference_layout(uint32_t* A_dst, const uint32_t* A_ref, int m, int k, void* stream);
 
+/* Measurement aid (no counterpart in the reference): a plain streaming read of `bytes` at `src`,
+ * launched like the decode kernels.  Its time on a buffer of a matrix's size is the ceiling that a
+ * launch, the first trip to HBM and the streaming itself set for a GEMM that reads the matrix once. */
+int w4a16_probe_read(w4a16_handle* h, const void* src, size_t bytes, void* stream);
+
 const char* w4a16_last_error(void);
 const char* w4a16_version(void);
 

@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libw4a16.so")
 
-SOURCES = ["api.cpp", "repack.hip", "static_scratch.hip", "gemm_decode.hip", "gemm_strip.hip", "gemm_sequence.hip", "gemm_prefill.hip"]
+SOURCES = ["api.cpp", "repack.hip", "static_scratch.hip", "probe.hip", "gemm_decode.hip", "gemm_strip.hip", "gemm_sequence.hip", "gemm_prefill.hip"]
 
 # -packed-fp32-ops off: hipcc must not form v_pk_*_f32 instructions for this target.
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
@@ -100,7 +100,7 @@ def build_library(verbose: bool = True) -> str:
     obj_dir = os.path.join(HERE, "build")
     os.makedirs(obj_dir, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(7, len(SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
         objs = list(ex.map(lambda s: _compile(s, obj_dir), SOURCES))
     tmp = LIB_PATH + ".tmp"
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]

@@ -646,6 +646,17 @@ int w4a16_from_reference_layout(uint32_t* A_dst, const uint32_t* A_ref, int m, i
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "from_reference_layout");
 }
 
+int w4a16_probe_read(w4a16_handle* h, const void* src, size_t bytes, void* stream)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    if (!src || !aligned16(src)) return fail(W4A16_EARG, "probe_read: src must be a 16-byte aligned device pointer");
+    // the sink (one word per workgroup, practically never written) is the unused tail of the barrier area
+    static_assert(kSyncInts - 64 * 40 >= 8 * 256, "no room for the probe's sink");
+    if (h->cus > 256) return fail(W4A16_ESHAPE, "probe_read: more than 256 CUs");
+    const hipError_t e = launch_probe_read(src, bytes, h->sync + 64 * 40, h->cus, (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "probe_read");
+}
+
 const char* w4a16_last_error(void)
 {
     return g_err;

@@ -110,6 +110,9 @@ hipError_t launch_fuse_w1_w3(uint32_t* dst, const uint32_t* src, int m, int k, h
 hipError_t launch_transpose_qk(uint32_t* dst, const uint32_t* src, int m, int k, int size_per_head, hipStream_t st);
 hipError_t launch_from_reference(uint32_t* dst, const uint32_t* ref, int m, int k, hipStream_t st);
 
+// measurement aid (probe.hip): a plain streaming read of `bytes`; sink = at least 8 * cus words
+hipError_t launch_probe_read(const void* src, size_t bytes, void* sink, int cus, hipStream_t st);
+
 // decode (skinny) kernels
 bool       decode_feasible(const DecodeConfig& cf, int N, int T, int K);
 size_t     decode_scratch_bytes(const DecodeConfig& cf, int N, int T, int K, size_t ws_bytes, int cnt_len);

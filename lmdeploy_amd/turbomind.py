@@ -163,6 +163,10 @@ class GemmS4F16:
     def set_barrier_timeout(self, seconds: float) -> None:
         check(lib.w4a16_set_barrier_timeout(self._h, seconds))
 
+    def probe_read(self, t, stream: Optional[int] = None) -> None:
+        """Measurement aid: a plain streaming read of tensor `t`, launched like the decode kernels."""
+        check(lib.w4a16_probe_read(self._h, _ptr(t), t.numel() * t.element_size(), _stream() if stream is None else stream))
+
     def pick(self, m: int, n: int, k: int) -> int:
         """The algo_id that `Run(..., algo_id=-1)` uses for this shape: the fastest one a previous
         `Measure` of exactly this shape found, else the heuristic's choice."""
