@@ -198,6 +198,25 @@ int w4a16_convert_s4_k_m8(uint32_t* A_dst, void* Q_dst, void* workspace, const u
                           const void* scales, const uint32_t* qzeros, int m, int k, int group_size,
                           void* stream);
 
+/* The fused q|k|v matrix of a decoder layer, straight from the three AWQ tensors of the checkpoint:
+ * what deploy_awq does with transpose_qk_s4 on q and k (lmdeploy/serve/turbomind/deploy.py:633-639;
+ * scales by `permute`, :371-383), merge_qkv (:251-260) and convert_s4 (:660-670), in one gather.
+ * qweight[i] uint32 [k, n_i/8], qzeros[i] uint32 [k/128, n_i/8], scales[i] fp16 [k/128, n_i] for
+ * i = q, k, v with n = n_q, n_kv, n_kv.  Within every head of size_per_head columns of q and k,
+ * output column 2i + r is source column r * size_per_head/2 + i.  A_dst: k * (n_q + 2 n_kv) / 2
+ * bytes, Q_dst: half2 [k/128, n_q + 2 n_kv]. */
+int w4a16_deploy_qkv(uint32_t* A_dst, void* Q_dst, const uint32_t* const qweight[3], const uint32_t* const qzeros[3],
+                     const void* const scales[3], int n_q, int n_kv, int k, int size_per_head, int group_size,
+                     void* stream);
+
+/* The fused gate|up matrix (w13) from the AWQ tensors of gate_proj (w1) and up_proj (w3): what
+ * deploy_awq does with fuse_w1_w3_s4 (deploy.py:641-658: output column 2j = w1 column j, 2j + 1 =
+ * w3 column j, for weights, zeros and scales) and convert_s4 (:660-670), in one gather.
+ * A_dst: k * 2 * inter_size / 2 bytes, Q_dst: half2 [k/128, 2 * inter_size]. */
+int w4a16_deploy_w13(uint32_t* A_dst, void* Q_dst, const uint32_t* w1_qweight, const uint32_t* w3_qweight,
+                     const uint32_t* w1_qzeros, const uint32_t* w3_qzeros, const void* w1_scales, const void* w3_scales,
+                     int inter_size, int k, int group_size, void* stream);
+
 /* reformat_s4_k_m8 (format.h:13, format.cu:69-75): the weight half of the conversion alone,
  * AWQ words [k, m/8] -> the tiled layout the GEMM kernels read (here the gfx950 one).
  * format.h:11 `reformat_s4_k8_m` is an unused alternative layout and has no counterpart. */

@@ -54,6 +54,9 @@ SIGNATURES = {
     "w4a16_pick": (c_int, [c_void_p, c_int, c_int, c_int]),
     "w4a16_clear_tuning": (c_int, [c_void_p]),
     "w4a16_convert_s4_k_m8": (c_int, [c_void_p] * 6 + [c_int] * 3 + [c_void_p]),
+    "w4a16_deploy_qkv": (c_int, [c_void_p, c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p)] + [c_int] * 5
+                         + [c_void_p]),
+    "w4a16_deploy_w13": (c_int, [c_void_p] * 8 + [c_int] * 3 + [c_void_p]),
     "w4a16_reformat_s4_k_m8": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "w4a16_fuse_w1_w3_s4_k_m8": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "w4a16_transpose_qk_s4_k_m8_hf": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),

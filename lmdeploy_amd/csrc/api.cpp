@@ -577,6 +577,47 @@ int w4a16_convert_s4_k_m8(uint32_t* A_dst, void* Q_dst, void* workspace, const u
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "convert_s4_k_m8");
 }
 
+int w4a16_deploy_qkv(uint32_t* A_dst, void* Q_dst, const uint32_t* const qweight[3], const uint32_t* const qzeros[3],
+                     const void* const scales[3], int n_q, int n_kv, int k, int size_per_head, int group_size, void* stream)
+{
+    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
+    if (n_q < 0 || n_kv < 0 || k < 0) return fail(W4A16_EARG, "deploy_qkv: negative size");
+    if (size_per_head <= 0 || size_per_head % 2 != 0 || n_q % size_per_head != 0 || n_kv % size_per_head != 0)
+        return fail(W4A16_ESHAPE, "deploy_qkv: q and k widths must be multiples of an even size_per_head");
+    if (n_q % 8 != 0 || n_kv % 8 != 0) return fail(W4A16_ESHAPE, "deploy_qkv: widths must be multiples of 8");
+    if (int c = check_repack("deploy_qkv", n_q + 2 * n_kv, k, 16, 128)) return c;
+    if (n_q + 2 * n_kv == 0 || k == 0) return W4A16_OK;
+    if (!A_dst || !Q_dst || !qweight || !qzeros || !scales) return fail(W4A16_EARG, "deploy_qkv: null pointer");
+    const int       width[3]  = {n_q, n_kv, n_kv};
+    const int       rotary[3] = {size_per_head, size_per_head, 0};
+    const uint16_t* s[3];
+    for (int i = 0; i < 3; ++i) {
+        if (width[i] > 0 && (!qweight[i] || !qzeros[i] || !scales[i])) return fail(W4A16_EARG, "deploy_qkv: null pointer");
+        s[i] = (const uint16_t*)scales[i];
+    }
+    const hipError_t e = launch_deploy(A_dst, (uint32_t*)Q_dst, qweight, qzeros, s, width, rotary, 0, k, (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "deploy_qkv");
+}
+
+int w4a16_deploy_w13(uint32_t* A_dst, void* Q_dst, const uint32_t* w1_qweight, const uint32_t* w3_qweight,
+                     const uint32_t* w1_qzeros, const uint32_t* w3_qzeros, const void* w1_scales, const void* w3_scales,
+                     int inter_size, int k, int group_size, void* stream)
+{
+    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
+    if (inter_size < 0 || k < 0) return fail(W4A16_EARG, "deploy_w13: negative size");
+    if (int c = check_repack("deploy_w13", inter_size, k, 8, 128)) return c;
+    if (inter_size == 0 || k == 0) return W4A16_OK;
+    if (!A_dst || !Q_dst || !w1_qweight || !w3_qweight || !w1_qzeros || !w3_qzeros || !w1_scales || !w3_scales)
+        return fail(W4A16_EARG, "deploy_w13: null pointer");
+    const uint32_t* qw[3]     = {w1_qweight, w3_qweight, nullptr};
+    const uint32_t* qz[3]     = {w1_qzeros, w3_qzeros, nullptr};
+    const uint16_t* s[3]      = {(const uint16_t*)w1_scales, (const uint16_t*)w3_scales, nullptr};
+    const int       width[3]  = {inter_size, inter_size, 0};
+    const int       rotary[3] = {0, 0, 0};
+    const hipError_t e = launch_deploy(A_dst, (uint32_t*)Q_dst, qw, qz, s, width, rotary, 1, k, (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "deploy_w13");
+}
+
 int w4a16_reformat_s4_k_m8(uint32_t* dst, const uint32_t* src, int m, int k, void* stream)
 {
     if (int c = check_repack("reformat_s4_k_m8", m, k, 16, 128)) return c;

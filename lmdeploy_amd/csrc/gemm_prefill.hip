@@ -525,7 +525,7 @@ struct Variant {
 // (a 256 x 256 tile does not fit the register file without spilling, and spill stores would
 // break the counted waits: stores and loads complete out of order with each other)
 constexpr Variant kVariants[] = {
-    {8, 2, 8, 2, 1, true, {1.905f, 3.821f, 5.517f, 7.090f, 13.658f}},   // 128 x 256, eight waves
+    {8, 2, 8, 2, 1, true, {1.810f, 3.630f, 5.240f, 6.740f, 12.980f}},   // 128 x 256, eight waves
     {16, 2, 4, 2, 1, true, {2.071f, 4.498f, 6.126f, 8.397f, 15.010f}},  // 256 x 128
     {8, 2, 4, 2, 1, false, {1.016f, 1.860f, 3.067f, 4.002f, 7.185f}},   // 128 x 128
     {4, 2, 4, 4, 1, false, {0.672f, 1.111f, 1.664f, 2.271f, 4.773f}},   //  64 x 128

@@ -64,6 +64,71 @@ merge_q_kernel(uint32_t* __restrict__ Q, const uint16_t* __restrict__ scales,
     Q[i]             = (0x5400u | (z << 4)) | ((uint32_t)scales[i] << 16);
 }
 
+// The columns of a deployable matrix, gathered from up to three AWQ tensors of the checkpoint:
+// side by side (q | k | v, deploy.py:251-260 `merge_qkv`), optionally with the columns of every
+// head re-ordered for rotary embedding (dst column 2i + r of a head <- column r * D/2 + i:
+// deploy.py:371-383 `permute`, format.cu:115-121), or interleaved in pairs (gate, up:
+// deploy.py:641-658 `fuse_w1_w3_s4`, format.cu:123-130).
+struct ColumnSource {
+    const uint32_t* qw[3];
+    const uint32_t* qz[3];
+    const uint16_t* s[3];
+    int             width[3];   // columns of each source
+    int             rotary[3];  // head size if the block's columns are re-ordered, else 0
+    int             interleave; // 1: column n comes from source n & 1, column n >> 1
+};
+struct Located {
+    int src, col;
+};
+__device__ __forceinline__ Located locate(const ColumnSource& cs, int n)
+{
+    if (cs.interleave) return Located{n & 1, n >> 1};
+    int b = 0;
+    while (b < 2 && n >= cs.width[b]) n -= cs.width[b++];
+    if (const int D = cs.rotary[b]) {
+        const int j = n % D;
+        n           = n - j + (j & 1) * (D / 2) + (j >> 1);
+    }
+    return Located{b, n};
+}
+
+// A_dst word `w` <- 8 rows of one column, taken from wherever the column lives
+__global__ void __launch_bounds__(kThreads)
+deploy_weights_kernel(uint32_t* __restrict__ dst, const ColumnSource cs, int N, int K)
+{
+    const int64_t w     = global_id();
+    const int64_t words = (int64_t)N * K / 8;
+    if (w >= words) return;
+    const int     NT   = N / kTileN;
+    const int     j    = (int)(w & 3);
+    const int     lane = (int)((w >> 2) & 63);
+    const int64_t tile = w >> 8;
+    const int     kt   = (int)(tile / NT);
+    const int     nt   = (int)(tile % NT);
+    const Located at   = locate(cs, nt * kTileN + (lane & 15));
+    const int     k0   = kt * kGroup + 32 * j + 8 * (lane >> 4);
+    const int     ld   = cs.width[at.src] / 8;
+    const uint32_t* src = cs.qw[at.src];
+    uint32_t      out  = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const uint32_t v = src[(int64_t)(k0 + e) * ld + (at.col >> 3)];
+        out |= awq_col(v, at.col & 7) << (4 * nibble_of_row(e));
+    }
+    dst[w] = out;
+}
+
+__global__ void __launch_bounds__(kThreads) deploy_q_kernel(uint32_t* __restrict__ Q, const ColumnSource cs, int N, int G)
+{
+    const int64_t i = global_id();
+    if (i >= (int64_t)N * G) return;
+    const int      g  = (int)(i / N);
+    const Located  at = locate(cs, (int)(i % N));
+    const int64_t  e  = (int64_t)g * cs.width[at.src] + at.col;
+    const uint32_t z  = awq_col(cs.qz[at.src][e >> 3], (int)(e & 7));
+    Q[i]              = (0x5400u | (z << 4)) | ((uint32_t)cs.s[at.src][e] << 16);
+}
+
 // inverse of repack_weights_kernel: one thread per AWQ word [k, n/8]
 __global__ void __launch_bounds__(kThreads)
 unrepack_weights_kernel(uint32_t* __restrict__ dst, const uint32_t* __restrict__ A, int N, int K)
@@ -241,6 +306,27 @@ hipError_t launch_convert(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* A_sr
     if (A_dst) e = launch_kernel(repack_weights_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, A_dst, A_src, m, k);
     if (Q_dst && e == hipSuccess)
         e = launch_kernel(merge_q_kernel, dim3(blocks_for(qn)), dim3(kThreads), 0, st, Q_dst, scales, qzeros, qn);
+    return e;
+}
+
+hipError_t launch_deploy(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* const qw[3], const uint32_t* const qz[3],
+                         const uint16_t* const s[3], const int width[3], const int rotary[3], int interleave, int k,
+                         hipStream_t st)
+{
+    ColumnSource cs{};
+    int          m = 0;
+    for (int i = 0; i < 3; ++i) {
+        cs.qw[i] = qw[i], cs.qz[i] = qz[i], cs.s[i] = s[i];
+        cs.width[i] = width[i], cs.rotary[i] = rotary[i];
+        m += width[i];
+    }
+    cs.interleave       = interleave;
+    const int64_t words = (int64_t)m * k / 8;
+    const int64_t qn    = (int64_t)(k / kGroup) * m;
+    if (words == 0) return hipSuccess;
+    hipError_t e = launch_kernel(deploy_weights_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, A_dst, cs, m, k);
+    if (e == hipSuccess)
+        e = launch_kernel(deploy_q_kernel, dim3(blocks_for(qn)), dim3(kThreads), 0, st, Q_dst, cs, m, k / kGroup);
     return e;
 }
 

@@ -101,6 +101,10 @@ hipError_t clear_counters(const Scratch& sc, hipStream_t st);
 
 hipError_t launch_convert(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* A_src, const uint16_t* scales,
                           const uint32_t* qzeros, int m, int k, hipStream_t st);
+// up to three AWQ tensors -> one deployable (A, Q): side by side, or (interleave) gate/up column pairs
+hipError_t launch_deploy(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* const qw[3], const uint32_t* const qz[3],
+                         const uint16_t* const s[3], const int width[3], const int rotary[3], int interleave, int k,
+                         hipStream_t st);
 hipError_t launch_unpack(uint32_t* qweight, uint32_t* qzeros, uint16_t* scales, const uint32_t* A,
                          const uint32_t* Q, int m, int k, hipStream_t st);
 hipError_t launch_dequantize_repacked(uint16_t* W, const uint32_t* A, const uint32_t* Q, int m, int k,

@@ -5,8 +5,9 @@ The W4A16 part of `deploy_awq` (`lmdeploy/serve/turbomind/deploy.py:554-783`) an
 loading of `loadWeights` (`src/turbomind/models/llama/LlamaDecoderLayerWeight.cc:207-218`).
 
 What is kept from the reference: tensor names (`model.layers.{i}.self_attn.q_proj.qweight` ...),
-the q/k rotary re-ordering (`transpose_qk_s4` on qweight and qzeros, `permute` on scales,
-`:371-383`), `merge_qkv` (`:251-260`), `fuse_w1_w3_s4` (`:641-658`), `convert_s4` (`:660-670`), the
+the result of its deploy steps - q/k rotary re-ordering (`:371-383`, `:633-639`), q|k|v side by side
+(`:251-260`), gate/up columns interleaved (`:641-658`), conversion (`:660-670`) - which the library
+computes per fused tensor in one gather (`w4a16_deploy_qkv`, `w4a16_deploy_w13`), the
 output file names `layers.{i}.attention.w_qkv.{rank}.qweight` / `.scales_zeros` (`:717-757`,
 `:172-192`) with their exact byte sizes (`.qweight` K*N/2, `.scales_zeros` K/128*N*4,
 `utils/memory_utils.cu:332-346`), and the `config.ini` keys `weight_type = int4`,
@@ -34,83 +35,33 @@ SIZE_PER_HEAD = 128
 
 
 # ---------------------------------------------------------------------------------------------
-# the W4A16 steps of deploy_awq, on GPU tensors
+# the W4A16 part of deploy_awq for one decoder layer
 # ---------------------------------------------------------------------------------------------
-def transpose_qk_s4(src: torch.Tensor, group_size: int = 128) -> torch.Tensor:
-    """deploy.py:633-639 (the reference passes group_size where the binding expects
-    size_per_head; both are 128)."""
-    assert src.is_contiguous()
-    dst = torch.empty_like(src)
-    tm.transpose_qk_s4_k_m8(src, dst, src.size(-1) * 8, src.size(0), group_size)
-    return dst
-
-
-def permute(x: torch.Tensor) -> torch.Tensor:
-    """deploy.py:371-383: interleaved rotary pairs -> half-split order, per head of 128."""
-    if x.shape[-1] > 1:
-        dim = x.shape[-1]
-        n_heads = dim // SIZE_PER_HEAD
-        return x.view(-1, n_heads, 2, dim // n_heads // 2).transpose(2, 3).reshape(-1, dim)
-    dim = x.shape[0]
-    n_heads = dim // SIZE_PER_HEAD
-    return x.view(n_heads, 2, dim // n_heads // 2, 1).transpose(1, 2).reshape(dim, 1)
-
-
-def merge_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, tp: int, dim: int) -> torch.Tensor:
-    """deploy.py:251-260."""
-    def reshape(x):
-        return x.view(x.size(0), tp, -1) if dim == 2 else x.view(tp, -1)
-    qkv = torch.cat((reshape(q), reshape(k), reshape(v)), dim=-1)
-    return qkv.view(q.size(0), -1)
-
-
-def fuse_w1_w3_s4(w1_qw, w1_qz, w1_s, w3_qw, w3_qz, w3_s):
-    """deploy.py:641-658: gate and up columns interleaved (weights, zeros and scales alike)."""
-    def fuse(a: torch.Tensor, b: torch.Tensor):
-        ab = torch.cat((a, b)).contiguous()
-        out = torch.empty_like(ab)
-        tm.fuse_w1_w3_s4_k_m8(ab, out, a.size(-1) * 8, a.size(0))
-        return out.view(a.size(0), -1)
-
-    w13_s = torch.cat((w1_s, w3_s)).view(2, w1_s.size(0), -1)
-    w13_s = w13_s.permute(1, 2, 0).contiguous().view(w1_s.size(0), -1)
-    return fuse(w1_qw, w3_qw), fuse(w1_qz, w3_qz), w13_s
-
-
-def convert_s4(qw: torch.Tensor, qz: torch.Tensor, s: torch.Tensor, group_size: int):
-    """deploy.py:660-670."""
-    assert qw.is_contiguous() and qz.is_contiguous() and s.is_contiguous()
-    A = torch.empty_like(qw)
-    Q = torch.empty_like(s, dtype=torch.int32)  # half2
-    tm.convert_s4_k_m8(A, Q, torch.empty(0, device=qw.device), qw, s, qz, qw.size(-1) * 8, qw.size(0), group_size)
-    return A, Q
-
-
 def convert_awq_layer(get: Callable[[str], torch.Tensor], i: int, group_size: int = 128) -> Dict[str, torch.Tensor]:
     """The int4 tensors of decoder layer `i` (deploy.py:676-757): `get(name)` returns the
-    checkpoint tensor of that name on the GPU.  Returns the eight deployable tensors keyed by the
-    reference's parameter names (without the rank infix)."""
-    p = "model.layers.%d." % i
-    att, mlp = p + "self_attn.", p + "mlp."
-    q_qw, k_qw, v_qw, o_qw = (get(att + n + "_proj.qweight") for n in "qkvo")
-    q_qz, k_qz, v_qz, o_qz = (get(att + n + "_proj.qzeros") for n in "qkvo")
-    q_s, k_s, v_s, o_s = (get(att + n + "_proj.scales") for n in "qkvo")
-    q_qw, k_qw = transpose_qk_s4(q_qw, group_size), transpose_qk_s4(k_qw, group_size)
-    q_qz, k_qz = transpose_qk_s4(q_qz, group_size), transpose_qk_s4(k_qz, group_size)
-    q_s, k_s = permute(q_s), permute(k_s)
+    checkpoint tensor of that name on the GPU, contiguous.  Returns the eight deployable tensors
+    keyed by the reference's parameter names (without the rank infix).  The library builds each fused
+    tensor in one pass from the checkpoint's tensors (`w4a16_deploy_qkv`, `w4a16_deploy_w13`); wo and
+    w2 need only the layout conversion."""
+    def awq(prefix: str):
+        return tuple(get(prefix + "." + part) for part in ("qweight", "qzeros", "scales"))
+
+    def plain(prefix: str):
+        qw, qz, s = awq(prefix)
+        A, Q = torch.empty_like(qw), torch.empty_like(s, dtype=torch.int32)   # Q: half2 per (group, feature)
+        tm.convert_s4_k_m8(A, Q, torch.empty(0, device=qw.device), qw, s, qz, qw.size(-1) * 8, qw.size(0), group_size)
+        return A, Q
+
+    att, mlp = "model.layers.%d.self_attn." % i, "model.layers.%d.mlp." % i
+    made = {"attention.w_qkv": tm.deploy_qkv(awq(att + "q_proj"), awq(att + "k_proj"), awq(att + "v_proj"),
+                                             SIZE_PER_HEAD, group_size),
+            "attention.wo": plain(att + "o_proj"),
+            "feed_forward.w13": tm.deploy_w13(awq(mlp + "gate_proj"), awq(mlp + "up_proj"), group_size),
+            "feed_forward.w2": plain(mlp + "down_proj")}
     out = {}
-    qkv = (merge_qkv(q_qw, k_qw, v_qw, 1, 2), merge_qkv(q_qz, k_qz, v_qz, 1, 2), merge_qkv(q_s, k_s, v_s, 1, 2))
-    out["layers.%d.attention.w_qkv.qweight" % i], out["layers.%d.attention.w_qkv.scales_zeros" % i] = \
-        convert_s4(*(t.contiguous() for t in qkv), group_size)
-    out["layers.%d.attention.wo.qweight" % i], out["layers.%d.attention.wo.scales_zeros" % i] = \
-        convert_s4(o_qw, o_qz, o_s, group_size)
-    w13 = fuse_w1_w3_s4(get(mlp + "gate_proj.qweight"), get(mlp + "gate_proj.qzeros"), get(mlp + "gate_proj.scales"),
-                        get(mlp + "up_proj.qweight"), get(mlp + "up_proj.qzeros"), get(mlp + "up_proj.scales"))
-    out["layers.%d.feed_forward.w13.qweight" % i], out["layers.%d.feed_forward.w13.scales_zeros" % i] = \
-        convert_s4(*(t.contiguous() for t in w13), group_size)
-    out["layers.%d.feed_forward.w2.qweight" % i], out["layers.%d.feed_forward.w2.scales_zeros" % i] = \
-        convert_s4(get(mlp + "down_proj.qweight"), get(mlp + "down_proj.qzeros"), get(mlp + "down_proj.scales"),
-                   group_size)
+    for key, (A, Q) in made.items():
+        out["layers.%d.%s.qweight" % (i, key)] = A
+        out["layers.%d.%s.scales_zeros" % (i, key)] = Q
     return out
 
 

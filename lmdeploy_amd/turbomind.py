@@ -59,6 +59,43 @@ def transpose_qk_s4_k_m8(src, dst, m: int, k: int, size_per_head: int) -> None:
     check(lib.w4a16_transpose_qk_s4_k_m8_hf(_ptr(dst), _ptr(src), m, k, size_per_head, _stream()))
 
 
+def deploy_qkv(q, k, v, size_per_head: int = 128, group_size: int = 128):
+    """The deployable fused q|k|v matrix from the checkpoint's AWQ tensors: q, k, v are
+    (qweight int32 [K, n/8], qzeros int32 [K/g, n/8], scales fp16 [K/g, n]) triples.  Does what
+    deploy_awq does with transpose_qk_s4 / permute, merge_qkv and convert_s4
+    (lmdeploy/serve/turbomind/deploy.py:251-260,371-383,633-639,660-670) in one pass; returns (A, Q)."""
+    K = q[0].size(0)
+    n_q, n_kv = q[0].size(-1) * 8, k[0].size(-1) * 8
+    if v[0].size(-1) * 8 != n_kv or any(t[0].size(0) != K for t in (k, v)):
+        raise ValueError("q, k, v shapes do not fit together")
+    for qw, qz, s in (q, k, v):
+        n = qw.size(-1) * 8
+        if qz.numel() * 8 != (K // group_size) * n or s.numel() != (K // group_size) * n:
+            raise ValueError("qzeros / scales shape does not match qweight")
+    n = n_q + 2 * n_kv
+    A = torch.empty((K, n // 8), dtype=torch.int32, device=q[0].device)
+    Q = torch.empty((K // group_size, n), dtype=torch.int32, device=q[0].device)
+    arr = lambda i: (ctypes.c_void_p * 3)(*(_ptr(t[i]) for t in (q, k, v)))
+    check(lib.w4a16_deploy_qkv(_ptr(A), _ptr(Q), arr(0), arr(1), arr(2), n_q, n_kv, K, size_per_head, group_size, _stream()))
+    return A, Q
+
+
+def deploy_w13(w1, w3, group_size: int = 128):
+    """The deployable fused gate|up matrix from the AWQ triples of gate_proj (w1) and up_proj (w3):
+    fuse_w1_w3_s4 + convert_s4 (deploy.py:641-670) in one pass; returns (A, Q)."""
+    K, n = w1[0].size(0), w1[0].size(-1) * 8
+    for a, b in zip(w1, w3):
+        if a.shape != b.shape:
+            raise ValueError("w1 and w3 shapes differ")
+    if w1[1].numel() * 8 != (K // group_size) * n or w1[2].numel() != (K // group_size) * n:
+        raise ValueError("qzeros / scales shape does not match qweight")
+    A = torch.empty((K, 2 * n // 8), dtype=torch.int32, device=w1[0].device)
+    Q = torch.empty((K // group_size, 2 * n), dtype=torch.int32, device=w1[0].device)
+    check(lib.w4a16_deploy_w13(_ptr(A), _ptr(Q), _ptr(w1[0]), _ptr(w3[0]), _ptr(w1[1]), _ptr(w3[1]), _ptr(w1[2]),
+                               _ptr(w3[2]), n, K, group_size, _stream()))
+    return A, Q
+
+
 def dequantize_s4(src, dst) -> None:
     """bind.cpp:458-465.  int32 words -> fp16 raw nibble values (8 per word)."""
     if src.numel() * 8 != dst.numel():

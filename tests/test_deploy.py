@@ -125,3 +125,40 @@ def test_reference_written_workspace_loads_into_the_same_tensors(tmp_path):
     assert np.array_equal(W.view(np.uint16), O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], G).view(np.uint16))
     with pytest.raises(ValueError, match="file size"):
         deploy.load_workspace_linear(str(wdir), "layers.0.attention.wo", K, N + 16)
+
+
+def test_fused_tensor_entry_points_equal_the_reference_steps_bit_for_bit():
+    """`w4a16_deploy_qkv` / `w4a16_deploy_w13` against the oracle's restatement of the reference's separate
+    steps (format.cu:115-130 on qweight and qzeros, deploy.py:371-383 and :651-652 on the scales, then
+    convert_s4_k_m8), with grouped-query widths (k and v narrower than q) and several heads."""
+    import lmdeploy_amd.turbomind as tm
+    rng = np.random.default_rng(77)
+    K, D = 512, 128
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a.view(np.int32) if a.dtype == np.uint32 else a)).cuda()
+
+    def rot_scales(s):       # deploy.py:371-377
+        g, dim = s.shape
+        return s.reshape(g, dim // D, 2, D // 2).transpose(0, 1, 3, 2).reshape(g, dim)
+
+    for n_q, n_kv in ((1024, 256), (256, 256)):
+        q, k, v = _awq(rng, K, n_q), _awq(rng, K, n_kv), _awq(rng, K, n_kv)
+        A, Q = tm.deploy_qkv(tuple(map(dev, q)), tuple(map(dev, k)), tuple(map(dev, v)), D)
+        qw = np.concatenate([O.transpose_qk_s4_k_m8_hf(q[0], n_q, K, D), O.transpose_qk_s4_k_m8_hf(k[0], n_kv, K, D), v[0]], axis=1)
+        qz = np.concatenate([O.transpose_qk_s4_k_m8_hf(q[1], n_q, K // G, D), O.transpose_qk_s4_k_m8_hf(k[1], n_kv, K // G, D),
+                             v[1]], axis=1)
+        s = np.concatenate([rot_scales(q[2]), rot_scales(k[2]), v[2]], axis=1)
+        N = n_q + 2 * n_kv
+        A_ref, Q_ref = O.convert_s4_k_m8(np.ascontiguousarray(qw), np.ascontiguousarray(s), np.ascontiguousarray(qz), N, K, G)
+        assert np.array_equal(A.cpu().numpy().view(np.uint32).reshape(-1), A_ref)
+        assert np.array_equal(Q.cpu().numpy().view(np.uint32), Q_ref)
+    F1 = 1408
+    w1, w3 = _awq(rng, K, F1), _awq(rng, K, F1)
+    A, Q = tm.deploy_w13(tuple(map(dev, w1)), tuple(map(dev, w3)))
+    qw = O.fuse_w1_w3_s4_k_m8(np.concatenate([w1[0], w3[0]]), F1, K)
+    qz = O.fuse_w1_w3_s4_k_m8(np.concatenate([w1[1], w3[1]]), F1, K // G)
+    s = np.stack([w1[2], w3[2]], axis=-1).reshape(K // G, 2 * F1)      # deploy.py:651-652
+    A_ref, Q_ref = O.convert_s4_k_m8(qw, np.ascontiguousarray(s), qz, 2 * F1, K, G)
+    assert np.array_equal(A.cpu().numpy().view(np.uint32).reshape(-1), A_ref)
+    assert np.array_equal(Q.cpu().numpy().view(np.uint32), Q_ref)
+    with pytest.raises(tm.W4A16Error):
+        tm.deploy_qkv(tuple(map(dev, q)), tuple(map(dev, k)), tuple(map(dev, v)), 96)     # 256 is not a multiple of 96
