@@ -94,9 +94,12 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-per-shape", action="store_true")
     ap.add_argument("--no-70b", action="store_true")
-    ap.add_argument("--probe", choices=["decode", "prefill", "decode-o"],
-                    help="run only the named kernel (gate_up decode / gate_up at T=2048 / o decode) plus a plain 256 MiB "
-                         "elementwise kernel, eagerly, for `rocprofv3 --pmc` (no JSON line)")
+    ap.add_argument("--probe", choices=["decode", "prefill", "decode-o", "sequence-trace"],
+                    help="decode / prefill / decode-o: run only the named kernel (gate_up decode / gate_up at T=2048 / o "
+                         "decode) plus a plain 256 MiB elementwise kernel, eagerly, for `rocprofv3 --pmc` (no JSON line).  "
+                         "sequence-trace: print the in-kernel time stamps of the persistent sequence kernel over Llama-2-7B "
+                         "layers at T=8 (needs W4A16_LIB=lmdeploy_amd/lib/libw4a16_trace.so from "
+                         "`python -m lmdeploy_amd.build --trace`)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -106,6 +109,10 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
+    trace = None
+    if args.probe == "sequence-trace":   # the tracing build reads the buffer's address from the environment at launch
+        trace = torch.zeros(4 * 256 * 8, dtype=torch.int64, device="cuda")
+        os.environ["W4A16_TRACE_PTR"] = "%x" % trace.data_ptr()
     import lmdeploy_amd.turbomind as tm
 
     torch.cuda.set_device(0)
@@ -119,7 +126,9 @@ def main():
     for name, K, N, epi in LAYER_7B:
         per_copy = K * N // 2 + (K // GROUP) * N * 4
         n = max(len(DECODE_T) * n_sets, N_LAYERS, int(args.cold_gib * 2 ** 30 / per_copy) + 1)
-        if args.probe:
+        if args.probe == "sequence-trace":
+            n = 16
+        elif args.probe:
             n = max(8, int(args.cold_gib * 2 ** 30 / per_copy) + 1) if name in ("gate_up", "o") else 1
         weights[name] = [make_weights(tm, torch, gen, name, K, N) for _ in range(n)]
     Tmax = max(max(DECODE_T), PREFILL_T)
@@ -162,6 +171,34 @@ def main():
             e1.record(stream)
             torch.cuda.synchronize()
         return e0.elapsed_time(e1)   # ms
+
+    if args.probe == "sequence-trace":
+        T, L = 8, 16
+        descs = []
+        for layer in range(L):
+            for name, K, N, epi in LAYER_7B:
+                A, Q = weights[name][layer]
+                descs.append((out[name], A, X[K], Q, N, K, epi, Res if epi == 2 else None, bool(descs)))
+        for rep in range(3):
+            for i in range(0, len(descs), 32):
+                gemm.sequence(descs[i:i + 32], T, persistent=True)
+            gemm.sequence_status()
+        t = trace.cpu().view(4, 256, 8).numpy()
+        if not t.any():
+            print("no time stamps: W4A16_LIB must name the tracing build (python -m lmdeploy_amd.build --trace)")
+            return
+        print("persistent sequence kernel, Llama-2-7B layers at T=8, second launch of 32 GEMMs; microseconds after the moment the "
+              "GEMM's inputs were ready (device-wide barrier passed), lane 0 of the named wave")
+        print("columns: first = first two groups multiplied | loop = K loop done | epi = sums reduced, outputs stored | "
+              "drained = stores written through | next = the next GEMM's inputs ready (its first weights were requested before the barrier)")
+        for who, label in enumerate(["workgroup 0 wave 0", "workgroup 0 wave 7", "workgroup 131 wave 0", "workgroup 131 wave 7"]):
+            print(label)
+            for u in range(8, 16):
+                r, nxt = t[who, u], t[who, u + 1]
+                f = lambda v: (v - r[0]) / 100.0
+                print("  %-8s first %5.2f | loop %5.2f | epi %5.2f | drained %5.2f | next %5.2f" % (
+                    LAYER_7B[u % 4][0], f(r[1]), f(r[2]), f(r[3]), f(nxt[4]), f(nxt[0])))
+        return
 
     if args.probe:
         # a plain elementwise kernel of known size calibrates FETCH_SIZE / WRITE_SIZE, then the kernel on cold weights
@@ -318,9 +355,22 @@ def main():
             torch.cuda.synchronize()
             dense_tf = 12 * flops(PREFILL_T, K, N) / e0.elapsed_time(e1) / 1e9
             del Wd, Y
-        ceilings = dict(reads, device_copy_512MiB_GBps=round(copy_gbs, 1),
+        barrier = {}
+        with torch.cuda.stream(stream):
+            for kind, tree in (("tree", True), ("single_counter", False)):
+                gemm.probe_barrier(200, tree)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                torch.cuda.synchronize()
+                e0.record(stream)
+                gemm.probe_barrier(2000, tree)
+                e1.record(stream)
+                torch.cuda.synchronize()
+                barrier[kind + "_us"] = round(e0.elapsed_time(e1) * 1e3 / 2000, 3)
+        gemm.sequence_status(stream.cuda_stream)
+        ceilings = dict(reads, device_wide_barrier=barrier, device_copy_512MiB_GBps=round(copy_gbs, 1),
                         dense_fp16_gemm_gate_up_T2048_TFLOPs=round(dense_tf, 1),
                         note="read_*: w4a16_probe_read (plain streaming read, one launch per buffer in a HIP graph, cold buffers); "
+                             "device_wide_barrier: w4a16_probe_barrier, one workgroup per CU, 2000 barriers in one launch; "
                              "torch copy_ (bytes read + written); torch.matmul fp16 (hipBLASLt)")
 
     # ---- Llama-2-70B layer shapes (BASELINE configs[3]) -----------------------------------------

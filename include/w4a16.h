@@ -256,6 +256,12 @@ int w4a16_from_reference_layout(uint32_t* A_dst, const uint32_t* A_ref, int m, i
  * launch, the first trip to HBM and the streaming itself set for a GEMM that reads the matrix once. */
 int w4a16_probe_read(w4a16_handle* h, const void* src, size_t bytes, void* stream);
 
+/* Measurement aid (no counterpart in the reference): one persistent launch of one workgroup per CU that
+ * crosses `iters` device-wide barriers of w4a16_gemm_sequence and does nothing else; time it with
+ * events and divide.  tree = 1: the two-level counter tree that the sequence kernel uses; tree = 0: every
+ * workgroup arrives on one counter. */
+int w4a16_probe_barrier(w4a16_handle* h, int iters, int tree, void* stream);
+
 const char* w4a16_last_error(void);
 const char* w4a16_version(void);
 

@@ -698,6 +698,14 @@ int w4a16_probe_read(w4a16_handle* h, const void* src, size_t bytes, void* strea
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "probe_read");
 }
 
+int w4a16_probe_barrier(w4a16_handle* h, int iters, int tree, void* stream)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    if (iters < 1 || iters > (1 << 20)) return fail(W4A16_EARG, "probe_barrier: iters out of range");
+    const hipError_t e = launch_probe_barrier(h->sync, iters, tree, h->cus, h->spin_ticks, (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "probe_barrier");
+}
+
 const char* w4a16_last_error(void)
 {
     return g_err;

@@ -156,7 +156,48 @@ __global__ void __launch_bounds__(64 * kWaves) sequence_kernel(const SeqArgs a)
     }
 }
 
+// Measurement aid: `iters` device-wide barriers and nothing else.  tree = 0 lets every workgroup arrive on
+// the root counter (what the two-level tree is there to avoid).
+__global__ void __launch_bounds__(64 * kWaves) barrier_probe_kernel(int* sync, int iters, int tree, long long spin_ticks)
+{
+    for (int no = 0; no < iters; ++no) {
+        if (threadIdx.x == 0) {
+            if (tree) {
+                grid_arrive_and_wait(sync, no, spin_ticks);
+            }
+            else {
+                const int old = __hip_atomic_fetch_add(sync_root(sync), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (old == (no + 1) * (int)gridDim.x - 1) {
+                    __hip_atomic_store(sync_flag(sync), no + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                else {
+                    const long long t0 = wall_clock64();
+                    while (__hip_atomic_load(sync_flag(sync), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) <= no &&
+                           wall_clock64() - t0 < spin_ticks)
+                        __builtin_amdgcn_s_sleep(1);
+                }
+            }
+        }
+        workgroup_barrier();
+    }
+    if (threadIdx.x == 0) {  // the last workgroup to leave puts the counters back to zero
+        const int old = __hip_atomic_fetch_add(sync_done(sync), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (old == (int)gridDim.x - 1) {
+            for (int l = 0; l < kLeaves; ++l) __hip_atomic_store(sync_leaf(sync, l), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(sync_root(sync), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(sync_flag(sync), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(sync_done(sync), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 }  // namespace
+
+hipError_t launch_probe_barrier(int* sync, int iters, int tree, int cus, long long spin_ticks, hipStream_t st)
+{
+    if (!sync || iters < 1 || cus < 1) return hipErrorInvalidValue;
+    return launch_kernel(barrier_probe_kernel, dim3(cus), dim3(64 * kWaves), 0, st, sync, iters, tree, spin_ticks);
+}
 
 bool sequence_feasible(const SeqGemm* g, int count, int T)
 {

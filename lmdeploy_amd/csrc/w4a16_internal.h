@@ -148,6 +148,9 @@ int        sequence_error_index();  // index of the error word in the sync area
 // `cus` workgroups (one per CU: they must all be resident at once); `spin_ticks` bounds each barrier wait
 hipError_t sequence_launch(const SeqGemm* g, int count, int T, int* sync, int cus, long long spin_ticks, hipStream_t st);
 
+// measurement aid: `iters` device-wide barriers of `cus` workgroups (tree = 0: all arrivals on one counter)
+hipError_t launch_probe_barrier(int* sync, int iters, int tree, int cus, long long spin_ticks, hipStream_t st);
+
 // MFMA prefill kernels
 int        prefill_variants();
 void       prefill_tile(int variant, int& tile_n, int& tile_t);

@@ -204,6 +204,10 @@ class GemmS4F16:
         """Measurement aid: a plain streaming read of tensor `t`, launched like the decode kernels."""
         check(lib.w4a16_probe_read(self._h, _ptr(t), t.numel() * t.element_size(), _stream() if stream is None else stream))
 
+    def probe_barrier(self, iters: int, tree: bool = True, stream: Optional[int] = None) -> None:
+        """Measurement aid: one persistent launch that crosses `iters` device-wide barriers and nothing else."""
+        check(lib.w4a16_probe_barrier(self._h, iters, int(tree), _stream() if stream is None else stream))
+
     def pick(self, m: int, n: int, k: int) -> int:
         """The algo_id that `Run(..., algo_id=-1)` uses for this shape: the fastest one a previous
         `Measure` of exactly this shape found, else the heuristic's choice."""
