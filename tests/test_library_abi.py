@@ -109,3 +109,51 @@ def test_build_module_imports_without_the_library():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True)
     assert r.returncode == 0, r.stderr
+
+
+def test_static_and_sequence_argument_validation(L):
+    lib = L.lib
+    # w4a16_gemm_static: the checks of w4a16_gemm, without a handle
+    s = lib.w4a16_gemm_static
+    assert s(P, P, P, P, None, 64, 4, 256, 64, 0, -1, None) == L.EGROUP and err(L) == "unsupported group size"
+    assert s(P, P, P, P, None, 72, 4, 256, 128, 0, -1, None) == L.ESHAPE
+    assert s(None, P, P, P, None, 64, 4, 256, 128, 0, -1, None) == L.EARG
+    assert s(P, P, P, P, None, 64, 4, 256, 128, 2, -1, None) == L.EARG and "residual" in err(L)
+    assert s(P, P, P, P, None, 64, 4, 256, 128, 0, 10 ** 6, None) == L.EALGO
+    assert s(None, None, None, None, None, 64, 0, 256, 128, 0, -1, None) == L.OK
+    # w4a16_gemm_sequence: every descriptor is validated before anything is launched
+    seq = lib.w4a16_gemm_sequence
+    one = (L.GemmDesc * 2)()
+    for d in one:
+        d.C, d.A, d.X, d.Q, d.R, d.n_out, d.k, d.epilogue, d.depends = 0x2000, 0x2000, 0x2000, 0x2000, None, 64, 256, 0, 1
+    assert seq(None, one, 2, 4, 128, 0, None) == L.EARG and "null handle" in err(L)
+    assert seq(FAKE, None, 2, 4, 128, 0, None) == L.EARG
+    assert seq(FAKE, one, 2, 4, 128, 8, None) == L.EARG and "flags" in err(L)
+    assert seq(FAKE, one, 2, 4, 64, 0, None) == L.EGROUP
+    one[1].n_out = 72
+    assert seq(FAKE, one, 2, 4, 128, L.SEQ_PERSISTENT, None) == L.ESHAPE
+    one[1].n_out, one[1].epilogue = 64, 2
+    assert seq(FAKE, one, 2, 4, 128, 0, None) == L.EARG and "residual" in err(L)
+    assert seq(FAKE, one, 0, 4, 128, 0, None) == L.OK            # empty list
+    one[1].epilogue = 0
+    assert seq(FAKE, one, 2, 0, 128, L.SEQ_PERSISTENT, None) == L.OK   # no tokens
+    assert lib.w4a16_set_barrier_timeout(None, 1.0) == L.EARG
+    assert lib.w4a16_sequence_status(None, None) == L.EARG
+    assert lib.w4a16_probe_read(None, P, 1024, None) == L.EARG
+    assert lib.w4a16_probe_barrier(None, 10, 1, None) == L.EARG
+
+
+def test_deploy_entry_point_validation(L):
+    lib = L.lib
+    three = (ctypes.c_void_p * 3)(0x2000, 0x2000, 0x2000)
+    q = lib.w4a16_deploy_qkv
+    assert q(P, P, three, three, three, 256, 256, 256, 128, 64, None) == L.EGROUP
+    assert q(P, P, three, three, three, 256, 256, 256, 96, 128, None) == L.ESHAPE      # 256 % 96
+    assert q(P, P, three, three, three, 256, 256, 200, 128, 128, None) == L.ESHAPE     # k % 128
+    assert q(None, P, three, three, three, 256, 256, 256, 128, 128, None) == L.EARG
+    assert q(P, P, (ctypes.c_void_p * 3)(0x2000, None, 0x2000), three, three, 256, 256, 256, 128, 128, None) == L.EARG
+    assert q(None, None, None, None, None, 0, 0, 256, 128, 128, None) == L.OK          # empty
+    w = lib.w4a16_deploy_w13
+    assert w(P, P, P, P, P, P, P, P, 64, 256, 32, None) == L.EGROUP
+    assert w(P, P, P, P, P, P, P, P, 60, 256, 128, None) == L.ESHAPE                   # inter_size % 8
+    assert w(P, P, P, None, P, P, P, P, 64, 256, 128, None) == L.EARG
