@@ -32,12 +32,13 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16 matrix
 
-# HBM bytes per launch of the two dominant kernels, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
+# HBM bytes per launch of the two dominant kernels and of the o decode kernel, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
 # runs of `bench.py --probe ...`, calibrated against an elementwise kernel of known size
 # (profiles/decode_gate_up_hbm_traffic.md, profiles/prefill_gate_up_mfma_and_traffic.md).
 N_LAYERS = 32          # Llama-2-7B
-TRAFFIC_DECODE_GATE_UP = 49.37e6
-TRAFFIC_PREFILL_GATE_UP = 565.2e6
+TRAFFIC_DECODE_GATE_UP = 49.36e6
+TRAFFIC_DECODE_O = 10.02e6
+TRAFFIC_PREFILL_GATE_UP = 567.7e6
 
 # name, K, N (gate_up: both halves), epilogue
 LAYER_7B = [("qkv", 4096, 12288, 0), ("o", 4096, 4096, 0), ("gate_up", 4096, 22016, 1), ("down", 11008, 4096, 2)]
@@ -242,7 +243,7 @@ def main():
     # ---- rooflines: the dominant decode kernel (gate_up) and the one furthest below its roofline (o) ----
     roofline = decode_roofline("gate_up", TRAFFIC_DECODE_GATE_UP,
                                "strip_kernel, gate_up K=4096 N=22016 +SiLU, T cycling over {1,4,8,16}")
-    roofline_worst = decode_roofline("o", None, "strip_kernel, o K=4096 N=4096, T cycling over {1,4,8,16}")
+    roofline_worst = decode_roofline("o", TRAFFIC_DECODE_O, "strip_kernel, o K=4096 N=4096, T cycling over {1,4,8,16}")
 
     # ---- per-shape decode table ----------------------------------------------------------------
     per_shape = []
