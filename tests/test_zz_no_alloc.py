@@ -88,3 +88,38 @@ def test_static_scratch_rejects_what_does_not_fit():
     with pytest.raises(tm.W4A16Error) as e:
         tm.gemm_static(C, A, X, Q, N, T, K, 64)
     assert e.value.code == -1
+
+
+def test_static_scratch_entry_point_under_graph_capture():
+    """The reason the entry point exists: it can be recorded into a HIP graph by a caller that has no handle and
+    has allocated nothing.  A graph holding split-K launches (their counters are cleared by a fill kernel, not a
+    memset node) is replayed several times with new activations written eagerly in between; every replay must equal
+    the eager result bit for bit."""
+    import lmdeploy_amd.turbomind as tm
+    K, N, T = 2176, 512, 40
+    d = O.make_inputs(5170, T, K, N, residual=True)
+    A, Q = convert(tm, d, N, K)
+    X, R = dev(d["X"]), dev(d["R"])
+    algos = [a for a, _ in split_k_algos(tm.GemmS4F16(), A, Q, X, N, T, K)][:4] + [-1]
+    outs = [torch.empty((T, N), dtype=torch.float16, device="cuda") for _ in algos]
+    tm.gemm_static(outs[0], A, X, Q, N, T, K, 128, tm.GemmS4F16.kFusedAdd, -1, residual=R)   # first call on the device: outside capture
+    stream = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=stream):
+        st = torch.cuda.current_stream().cuda_stream
+        for a, C in zip(algos, outs):
+            tm.gemm_static(C, A, X, Q, N, T, K, 128, tm.GemmS4F16.kFusedAdd, a, residual=R, stream=st)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(11)
+    for rep in range(4):
+        X.copy_(torch.randn((T, K), device="cuda", generator=gen).half())
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for a, C in zip(algos, outs):
+            E = torch.empty_like(C)
+            tm.gemm_static(E, A, X, Q, N, T, K, 128, tm.GemmS4F16.kFusedAdd, a, residual=R)
+            torch.cuda.synchronize()
+            assert torch.equal(E.view(torch.int16), C.view(torch.int16)), (rep, a)
+    want = O.gemm_s4_f16(X.cpu().numpy(), d["qweight"], d["qzeros"], d["scales"], 128, O.EPI_ADD, d["R"])
+    assert O.max_abs_rel(outs[-1].cpu().numpy(), want) <= TOL
