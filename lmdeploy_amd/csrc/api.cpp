@@ -165,7 +165,7 @@ int algo_pick(int N, int T, int K, const Scratch& lim)
         const double blocks    = (T + 15) / 16;
         const double decode_us = 3.0 + std::pow(blocks, 0.85) * ((double)K * N / 2) / 4.2e6 * (N / 16 < 512 ? 1.4 : 1.0);
         // 17..32 tokens: the strip kernel with 32 tokens per workgroup streams the weights once, at
-        // 1.25 x (17 tokens) to 1.6 x (32 tokens) the cost of a 16-token pass
+        // 1.2 x (17 tokens) to 1.4 x (32 tokens) the cost of a 16-token pass
         int    strip32 = -1;
         double strip32_us = 0;
         if (T <= 32) {
@@ -173,7 +173,7 @@ int algo_pick(int N, int T, int K, const Scratch& lim)
                 const Algo& a = algo_at(id);
                 if (a.kind == 2 && a.tile_t == 32 && a.param == 1 && algo_feasible(id, N, T, K, lim)) strip32 = id;
             }
-            strip32_us = 3.0 + (1.25 + 0.35 * (T - 16) / 16.0) * ((double)K * N / 2) / 4.2e6;
+            strip32_us = 3.0 + (1.2 + 0.2 * (T - 16) / 16.0) * ((double)K * N / 2) / 4.2e6;
         }
         if (best >= 0 && best_us < decode_us && (strip32 < 0 || best_us < strip32_us)) return best;
         if (strip32 >= 0 && strip32_us < decode_us) return strip32;

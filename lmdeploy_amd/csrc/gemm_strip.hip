@@ -15,6 +15,12 @@
 // cost more than a third of the kernel; (c) two groups are in
 // flight per wave from its first instruction on (2 R + 8 KiB).
 //
+// With 32 tokens per workgroup (17 to 32 tokens) every workgroup still reads all of the activations
+// once, which is then several times the weight bytes of a narrow strip: the activations of a group go
+// from memory straight into the wave's LDS patch (no registers), which leaves registers for strips of
+// up to eight tiles, so that one workgroup per CU suffices on the widest matrices and the activations
+// are read 256 times instead of 512.
+//
 // Arithmetic per group and tile is that of the column-block decode kernel: four MFMAs on the
 // unpacked int4 still carrying its fp16 offset, four on a B operand of -(offset + z), then
 // acc += s * sum in fp32.
@@ -32,7 +38,7 @@ using namespace strip;
 template<int RMAX, int TP, int EPI>
 __global__ void __launch_bounds__(64 * kWaves) strip_kernel(const StripParams p)
 {
-    extern __shared__ __attribute__((aligned(16))) u32x4_t smem[];  // activation patches [8][TP][16], then sums [8][R][64]
+    extern __shared__ __attribute__((aligned(16))) u32x4_t smem[];  // activation patches [8][1 or 2][TP][16], then sums [8][R][H][64]
     const int bx   = blockIdx.x;
     const bool wide = bx < p.rem;
     const int col0 = bx * p.base + min(bx, p.rem);
@@ -49,11 +55,22 @@ template<int RMAX, int TP>
 hipError_t launch_rt(const StripParams& p, dim3 grid, size_t lds, int epilogue, hipStream_t st)
 {
     const dim3 block(64 * kWaves);
+#define W4A16_LAUNCH(EPI)                                                                                              \
+    do {                                                                                                               \
+        auto kfn = strip_kernel<RMAX, TP, EPI>;                                                                        \
+        if constexpr (TP == 32) { /* up to 128 KiB of LDS: above the default limit */                                  \
+            static std::atomic<uint64_t> raised{0};                                                                    \
+            const hipError_t e = raise_lds_limit(reinterpret_cast<const void*>(kfn), 8 * kMaxR32 * 2 * 1024, raised);  \
+            if (e != hipSuccess) return e;                                                                             \
+        }                                                                                                              \
+        return launch_kernel(kfn, grid, block, lds, st, p);                                                            \
+    } while (0)
     switch (epilogue) {
-        case kEpiGemm: return launch_kernel(strip_kernel<RMAX, TP, kEpiGemm>, grid, block, lds, st, p);
-        case kEpiSilu: return launch_kernel(strip_kernel<RMAX, TP, kEpiSilu>, grid, block, lds, st, p);
-        default: return launch_kernel(strip_kernel<RMAX, TP, kEpiAdd>, grid, block, lds, st, p);
+        case kEpiGemm: W4A16_LAUNCH(kEpiGemm);
+        case kEpiSilu: W4A16_LAUNCH(kEpiSilu);
+        default: W4A16_LAUNCH(kEpiAdd);
     }
+#undef W4A16_LAUNCH
 }
 
 template<int RMAX>
@@ -119,13 +136,13 @@ hipError_t strip_launch(int per_cu, int block_t, const GemmArgs& a, hipStream_t 
 {
     const StripPlan pl = make_plan(per_cu, block_t, a.N, a.T, a.K);
     if (!pl.ok) return hipErrorInvalidValue;
-    const int   G  = a.K / kGroup;
     const int   tp = block_t == 32 ? 32 : (a.T <= 4 ? 4 : (a.T <= 8 ? 8 : 16));
     const int   h  = tp > 16 ? tp / 16 : 1;
     StripParams p{a.C, reinterpret_cast<const u32x4_t*>(a.A), a.X, a.Q, a.R, a.N, a.T, a.K, pl.base, pl.rem,
-                  (G + kWaves - 1) / kWaves, a.epilogue};
+                  0, a.epilogue};
     const dim3   grid(pl.strips, (a.T + block_t - 1) / block_t);
-    const size_t lds = (size_t)kWaves * std::max(pl.rmax * h * 1024, tp * 256);
+    // per wave: the sums of its strip, over its activation patch(es) - two for 32 tokens, which arrive straight from memory
+    const size_t lds = (size_t)kWaves * std::max(pl.rmax * h * 1024, tp * 256 * (tp >= kDmaTokens ? 2 : 1));
     switch (pl.rmax) {
         case 1: return launch_r<1>(tp, p, grid, lds, a.epilogue, st);
         case 2: return launch_r<2>(tp, p, grid, lds, a.epilogue, st);

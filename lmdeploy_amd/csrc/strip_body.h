@@ -22,8 +22,12 @@ namespace strip {
 
 constexpr int kWaves   = 8;  // = K slices per workgroup
 constexpr int kMaxR    = 8;  // column tiles per strip
-constexpr int kMaxR32  = 4;  // ... with 32 tokens per workgroup (register budget)
+constexpr int kMaxR32  = 8;  // ... with 32 tokens per workgroup
 constexpr int kNumCU   = 256;
+#ifndef W4A16_DMA_TOKENS
+#define W4A16_DMA_TOKENS 32
+#endif
+constexpr int kDmaTokens = W4A16_DMA_TOKENS;  // token block from which the activations go straight to LDS
 
 struct StripParams {
     uint16_t*       C;
@@ -34,7 +38,7 @@ struct StripParams {
     int             N, T, K;
     int             base;  // column tiles of a narrow strip
     int             rem;   // the first `rem` strips have base + 1
-    int             per;   // groups per slice = ceil(G / 8)
+    int             tag;   // not read by the kernels: the tracing build files its time stamps under this number
     int             epilogue;  // read by kernels whose epilogue is chosen at run time (EPI == kEpiRuntime)
 };
 
@@ -44,7 +48,6 @@ constexpr int kEpiRuntime = 3;  // template value: take the epilogue from StripP
 // `u`, recorded by lane 0 of waves 0 and 7 of two workgroups.
 #ifdef W4A16_TRACE
 static __device__ long long* g_trace;
-static __device__ int        g_trace_unit;
 #define W4A16_STAMP(slot)                                                                                              \
     do {                                                                                                               \
         if (g_trace && (threadIdx.x & 63) == 0 && ((threadIdx.x >> 6) == 0 || (threadIdx.x >> 6) == 7) &&              \
@@ -104,6 +107,28 @@ __device__ __forceinline__ void mload128_agent(u32x4_t& dst, uint32_t voff, cons
                  : "scc");
 }
 
+// Global memory straight into LDS (no registers): lane l's 16 bytes land at lds_base + 16 l.  The LDS
+// base travels in M0.  Counts in vmcnt like any other load, and is complete there when the data is in LDS.
+__device__ __forceinline__ uint32_t lds_addr(const void* p)
+{
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)(p);
+}
+__device__ __forceinline__ void mload128_lds(uint32_t lds_base, uint32_t voff, const void* sbase, int flag)
+{
+    uint64_t sv;
+    asm volatile("s_mov_b32 m0, %[lb]\n\t" W4A16_MASKED("global_load_lds_dwordx4 %[vo], %[sb]\n\t")
+                 : [sv] "=&s"(sv)
+                 : [vo] "v"(voff), [sb] "s"(sbase), [mk] "s"(flag), [lb] "s"(lds_base)
+                 : "scc", "m0", "memory");
+}
+// LDS fragment read from inline assembly: the compiler would put a wait for every load in flight in front of
+// an LDS read of its own that follows a direct-to-LDS load.
+template<int OFF>
+__device__ __forceinline__ void lds_read128(half8_t& dst, uint32_t addr)
+{
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+
 template<int I, int N, typename F>
 __device__ __forceinline__ void static_for(F&& f)
 {
@@ -119,7 +144,7 @@ template<int R, int NX>
 struct Stage {
     u32x4_t  w[R];
     uint32_t q[R];
-    u32x4_t  x[NX];
+    u32x4_t  x[NX > 0 ? NX : 1];  // (NX = 0: the activations go straight to LDS)
 };
 
 // The whole kernel for a strip of exactly R column tiles starting at tile `col0`.
@@ -147,7 +172,7 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     // H row blocks of 16 tokens share every unpacked weight (H = 2 for the 32-token variant)
     constexpr int H  = TP > 16 ? TP / 16 : 1;
     const int     t0 = SEQ ? 0 : blockIdx.y * (16 * H);
-    [[maybe_unused]] const int trace_unit = p.per;  // (sequence kernel: the unit's number travels in `per`)
+    [[maybe_unused]] const int trace_unit = p.tag;
     const int     Tl = min(16 * H, T - t0);
 
     // this wave's groups: wave, wave + 8, wave + 16, ...  Interleaved rather than blocked, so that
@@ -166,12 +191,22 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     // more than the weight stream.)  The wave turns the rows into operand order through a private
     // patch of LDS; chunk p of row r sits at position p ^ r so that both the row-wise writes and
     // the column-wise reads are free of bank conflicts.
-    constexpr int NX = TP / 4;
-    uint32_t      x_off[NX];
+    // With 32 tokens the rows go from global memory straight into the patch instead (no registers, no
+    // LDS write), one patch per group in flight; the swizzle is then applied on the way in: the lane
+    // that lands at position p of row r fetches chunk p ^ r.
+    constexpr int  D    = 2;  // groups in flight per wave
+    constexpr bool XDMA = TP >= kDmaTokens && !SEQ;
+    constexpr int  NX   = TP / 4;
+    constexpr int  NXR  = XDMA ? 0 : NX;  // activation loads that land in registers
+    uint32_t       x_off[NX];
 #pragma unroll
-    for (int i = 0; i < NX; ++i)
-        x_off[i] = (uint32_t)min(t0 + 4 * i + (lane >> 4), T - 1) * (uint32_t)(K * 2) + (uint32_t)((lane & 15) * 16);
-    u32x4_t* const xw = smem + wave * (TP * 16);  // this wave's patch: [TP rows][16 chunks]
+    for (int i = 0; i < NX; ++i) {
+        const int r     = 4 * i + (lane >> 4);
+        const int chunk = XDMA ? ((lane & 15) ^ (r & 15)) : (lane & 15);
+        x_off[i]        = (uint32_t)min(t0 + r, T - 1) * (uint32_t)(K * 2) + (uint32_t)(chunk * 16);
+    }
+    u32x4_t* const xw = smem + wave * (TP * 16) * (XDMA ? D : 1);  // this wave's patch(es): [TP rows][16 chunks]
+    const uint32_t xw_lds = __builtin_amdgcn_readfirstlane(lds_addr(xw));
     int            xw_at[NX], xr_at[H][4];
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
@@ -190,15 +225,17 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     const char* Qb = reinterpret_cast<const char*>(p.Q) + (int64_t)col0 * 64;
     const char* Xb = reinterpret_cast<const char*>(p.X);
 
-    // All loads of group g into stage s; enable = false turns them into no-ops that still count.
-    auto issue_x = [&](Stage<R, NX>& s, int g, bool enable) {
+    // All loads of group g into stage s (number d); enable = false turns them into no-ops that still count.
+    using StageT = Stage<R, NXR>;
+    auto issue_x = [&](StageT& s, int d, int g, bool enable) {
         const int flag = __builtin_amdgcn_readfirstlane(enable ? 1 : 0);
         static_for<0, NX>([&](auto i) {
-            if constexpr (SEQ) mload128_agent(s.x[i], x_off[i], Xb + (int64_t)g * 256, flag);
+            if constexpr (XDMA) mload128_lds(xw_lds + (uint32_t)(d * TP * 256 + i * 1024), x_off[i], Xb + (int64_t)g * 256, flag);
+            else if constexpr (SEQ) mload128_agent(s.x[i], x_off[i], Xb + (int64_t)g * 256, flag);
             else mload128(s.x[i], x_off[i], Xb + (int64_t)g * 256, flag);
         });
     };
-    auto issue_wq = [&](Stage<R, NX>& s, int g, bool enable) {
+    auto issue_wq = [&](StageT& s, int g, bool enable) {
         const int flag = __builtin_amdgcn_readfirstlane(enable ? 1 : 0);
         const char* qg = Qb + (int64_t)g * N * 4;
         static_for<0, R>([&](auto r) { mload32<r * 64>(s.q[r], q_off, qg, flag); });
@@ -208,8 +245,8 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
             mload128_nt<(r % 4) * 1024>(s.w[r], w_off, wg, flag);
         });
     };
-    auto issue = [&](Stage<R, NX>& s, int g, bool enable) {
-        issue_x(s, g, enable);
+    auto issue = [&](StageT& s, int d, int g, bool enable) {
+        issue_x(s, d, g, enable);
         issue_wq(s, g, enable);
     };
     constexpr int kLoads = 2 * R + NX;  // loads per stage
@@ -224,14 +261,32 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     // One tile of one group.  U tiles are worked on at a time with their MFMA chains interleaved:
     // a chain is eight dependent MFMAs, and a dependent MFMA cannot issue before its predecessor
     // has left the pipe.
-    auto compute = [&](Stage<R, NX>& s) {
+    auto compute = [&](StageT& s, auto dc) {
         half8_t xf[H][4];
+        if constexpr (XDMA) {
+            // the group's rows are in patch d: row block h is 4 KiB further on
+            constexpr int d = decltype(dc)::value;
+            static_for<0, H * 4>([&](auto hj) {
+                constexpr int h = decltype(hj)::value / 4, j = decltype(hj)::value % 4;
+                lds_read128<d * TP * 256 + h * 4096>(xf[h][j], xw_lds + (uint32_t)(xr_at[0][j] * 16));
+            });
+            // (every fragment exactly once: a register named twice would be copied before the wait)
+            static_assert(H <= 2, "the wait below names the fragments of at most two row blocks");
+            if constexpr (H == 1)
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xf[0][0]), "+v"(xf[0][1]), "+v"(xf[0][2]), "+v"(xf[0][3]));
+            else
+                asm volatile("s_waitcnt lgkmcnt(0)"
+                             : "+v"(xf[0][0]), "+v"(xf[0][1]), "+v"(xf[0][2]), "+v"(xf[0][3]), "+v"(xf[H - 1][0]),
+                               "+v"(xf[H - 1][1]), "+v"(xf[H - 1][2]), "+v"(xf[H - 1][3]));
+        }
+        else {
 #pragma unroll
-        for (int i = 0; i < NX; ++i) xw[xw_at[i]] = s.x[i];
+            for (int i = 0; i < NXR; ++i) xw[xw_at[i]] = s.x[i];
 #pragma unroll
-        for (int h = 0; h < H; ++h)
+            for (int h = 0; h < H; ++h)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) xf[h][j] = __builtin_bit_cast(half8_t, xw[xr_at[h][j]]);  // same wave: LDS keeps the order
+                for (int j = 0; j < 4; ++j) xf[h][j] = __builtin_bit_cast(half8_t, xw[xr_at[h][j]]);  // same wave: LDS keeps the order
+        }
         constexpr int U = 2;
 #pragma unroll
         for (int r0 = 0; r0 < R; r0 += U) {
@@ -290,17 +345,16 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     // Wait until the stage's loads are complete (loads return in order: at most `kLoads` younger
     // ones may still be in flight, or none after the last issue), then pin its registers below
     // the wait.
-    auto pin = [&](Stage<R, NX>& s) {
+    auto pin = [&](StageT& s) {
 #pragma unroll
         for (int r = 0; r < R; ++r) asm volatile("" : "+v"(s.w[r]), "+v"(s.q[r]));
 #pragma unroll
-        for (int i = 0; i < NX; ++i) asm volatile("" : "+v"(s.x[i]));
+        for (int i = 0; i < NXR; ++i) asm volatile("" : "+v"(s.x[i]));
     };
     // Two groups in flight per wave.  (Three or four fit the register file for narrow strips but
     // measured slower: the unrolled loop body grows with D and is executed only once or twice.)
-    constexpr int D = 2;
     static_assert((D - 1) * kLoads <= 63, "vmcnt is a 6-bit counter");
-    Stage<R, NX> st[D];
+    StageT st[D];
 #pragma unroll
     for (int d = 0; d < D; ++d) {
 #pragma unroll
@@ -309,18 +363,20 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
             st[d].q[r] = 0;
         }
 #pragma unroll
-        for (int i = 0; i < NX; ++i) st[d].x[i] = u32x4_t{0, 0, 0, 0};
+        for (int i = 0; i < NXR; ++i) st[d].x[i] = u32x4_t{0, 0, 0, 0};
     }
 
     // One group: wait for the stage (exactly D - 1 younger stages are in flight behind it), use
     // it, refill it.  Nothing of a stage may be live when it is refilled (the refill is in place
     // and asynchronous), so the scheduler must not move the stage's arithmetic below its refill.
-    auto step = [&](Stage<R, NX>& s, bool use, int refill_group, bool refill) {
+    auto step = [&](auto dc, bool use, int refill_group, bool refill) {
+        constexpr int d = decltype(dc)::value;
+        StageT&       s = st[d];
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((D - 1) * kLoads) : "memory");
         pin(s);
-        if (use) compute(s);
+        if (use) compute(s, dc);
         __builtin_amdgcn_sched_barrier(0);
-        issue(s, min(refill_group, G - 1), refill);
+        issue(s, d, min(refill_group, G - 1), refill);
     };
 
     if constexpr (SEQ) {
@@ -330,18 +386,20 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
         for (int d = 0; d < D; ++d) issue_wq(st[d], min(g0 + d * kStep, G - 1), d < cnt);
         inputs_ready();
 #pragma unroll
-        for (int d = 0; d < D; ++d) issue_x(st[d], min(g0 + d * kStep, G - 1), d < cnt);
+        for (int d = 0; d < D; ++d) issue_x(st[d], d, min(g0 + d * kStep, G - 1), d < cnt);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     else {
 #pragma unroll
-        for (int d = 0; d < D; ++d) issue(st[d], min(g0 + d * kStep, G - 1), d < cnt);
+        for (int d = 0; d < D; ++d) issue(st[d], d, min(g0 + d * kStep, G - 1), d < cnt);
     }
     // D groups per trip, so that each stage keeps its registers; all conditions are wave-uniform
     // and none of them surrounds a load.
     for (int i = 0; i < cnt; i += D) {
-#pragma unroll
-        for (int d = 0; d < D; ++d) step(st[d], i + d < cnt, g0 + (i + d + D) * kStep, i + d + D < cnt);
+        static_for<0, D>([&](auto dc) {
+            constexpr int d = decltype(dc)::value;
+            step(dc, i + d < cnt, g0 + (i + d + D) * kStep, i + d + D < cnt);
+        });
         if (i == 0) W4A16_STAMP(1);
     }
     W4A16_STAMP(2);

@@ -287,7 +287,8 @@ def test_strip_kernels_on_wide_matrices(tm, gemm, algo_table, N):
 
 @pytest.mark.parametrize("name,K,N,kind", [("qkv", 4096, 12288, 0), ("gate_up", 4096, 22016, 1)])
 def test_llama7b_wide_shapes_at_17_to_32_tokens_take_the_32_token_strips(tm, gemm, algo_table, name, K, N, kind):
-    """qkv (strips of 3 tiles) and gate_up (strips of 3 and 2: 512 workgroups) with 32 token rows per workgroup:
+    """qkv (strips of 3 tiles) and gate_up (strips of 6 and 5 on 256 workgroups, of 3 and 2 on 512) with 32 token
+    rows per workgroup, four groups per wave (so every LDS patch is refilled while the other one is in use):
     what the default dispatch picks at 17 and 24 tokens, and forced by id at 32 (where the dispatch may prefer
     an MFMA tile)."""
     d = O.make_inputs(4100 + kind, 32, K, N)
