@@ -95,12 +95,17 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-per-shape", action="store_true")
     ap.add_argument("--no-70b", action="store_true")
-    ap.add_argument("--probe", choices=["decode", "prefill", "decode-o", "sequence-trace"],
+    ap.add_argument("--seconds", type=float, default=8.0, help="duration of the sustain-* probes")
+    ap.add_argument("--probe", choices=["decode", "prefill", "decode-o", "sequence-trace", "sustain-prefill",
+                                        "sustain-decode", "sustain-dense"],
                     help="decode / prefill / decode-o: run only the named kernel (gate_up decode / gate_up at T=2048 / o "
                          "decode) plus a plain 256 MiB elementwise kernel, eagerly, for `rocprofv3 --pmc` (no JSON line).  "
                          "sequence-trace: print the in-kernel time stamps of the persistent sequence kernel over Llama-2-7B "
                          "layers at T=8 (needs W4A16_LIB=lmdeploy_amd/lib/libw4a16_trace.so from "
-                         "`python -m lmdeploy_amd.build --trace`)")
+                         "`python -m lmdeploy_amd.build --trace`).  sustain-prefill / sustain-decode / sustain-dense: "
+                         "keep launching gate_up (T=2048 / T=8 / torch.matmul fp16 at T=2048) for --seconds and print the "
+                         "rate once a second, so that the engine clock under that load can be read beside it "
+                         "(`rocm-smi --showclocks`)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -199,6 +204,33 @@ def main():
                 f = lambda v: (v - r[0]) / 100.0
                 print("  %-8s first %5.2f | loop %5.2f | epi %5.2f | drained %5.2f | next %5.2f" % (
                     LAYER_7B[u % 4][0], f(r[1]), f(r[2]), f(r[3]), f(nxt[4]), f(nxt[0])))
+        return
+
+    if args.probe and args.probe.startswith("sustain-"):
+        K, N, _ = shape["gate_up"]
+        T = 8 if args.probe == "sustain-decode" else PREFILL_T
+        dense_w = torch.randn(K, N, device="cuda", generator=gen).half() if args.probe == "sustain-dense" else None
+        dense_out = torch.empty(T, N, dtype=torch.float16, device="cuda") if dense_w is not None else None
+        n, per = len(weights["gate_up"]), 2000 if T == 8 else 200
+        t_end, t0, shown = time.time() + args.seconds, time.time(), -1
+        while time.time() < t_end:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            with torch.cuda.stream(stream):
+                e0.record()
+                for c in range(per):
+                    if dense_w is not None:
+                        torch.matmul(X[K][:T], dense_w, out=dense_out)
+                    else:
+                        launch("gate_up", c % n, T, stream.cuda_stream)
+                e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / per
+            if int(time.time() - t0) == shown:
+                continue
+            shown = int(time.time() - t0)
+            print("%s t=%4.1fs  %7.1f us/launch  %6.0f TFLOP/s  %6.0f GB/s" % (
+                args.probe, time.time() - t0, us, 2.0 * T * K * N / us / 1e6,
+                algorithmic_bytes(T, K, N, 0 if dense_w is not None else 1) / us / 1e3), flush=True)
         return
 
     if args.probe:
