@@ -61,7 +61,8 @@ typedef struct w4a16_metric {
  * w4a16_destroy.  That first launch must not be under graph capture: there, a handle that has no
  * workspace yet uses kernels that need none (algo_id < 0) or fails with W4A16_ESCRATCH (explicit
  * algo_id).  GEMMs issued through one handle must be ordered on one stream at a time, because they
- * share that scratch. */
+ * share that scratch.  A handle has no lock: one host thread uses it at a time.  Every call that
+ * launches through a handle checks that the handle's device is the current one (W4A16_EARG if not). */
 int  w4a16_create(w4a16_handle** out);
 void w4a16_destroy(w4a16_handle* h);
 

@@ -256,6 +256,18 @@ int check_prefill_alignment(int algo_id, const void* C, const void* R, int epilo
     return 0;
 }
 
+// A handle's scratch, counters and events live on the device that was current at w4a16_create; a launch
+// made with another device current would hand them to a GPU that cannot reach them.
+int check_device(const w4a16_handle* h)
+{
+    int              dev = -1;
+    const hipError_t e   = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    if (dev != h->device)
+        return fail(W4A16_EARG, "the handle belongs to device %d but device %d is current", h->device, dev);
+    return W4A16_OK;
+}
+
 // the kernel w4a16_gemm uses for algo_id < 0: a measured one if this exact shape was measured
 int pick_for(const w4a16_handle* h, int n_out, int tokens, int k)
 {
@@ -370,6 +382,7 @@ int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const voi
     if (chk < 0) return chk;
     if (chk > 0) return W4A16_OK;
     if (algo_id >= algo_count()) return fail(W4A16_EALGO, "algo_id %d out of range (0..%d)", algo_id, algo_count() - 1);
+    if (int rc = check_device(h)) return rc;
     const bool chosen = algo_id >= 0;
     if (!chosen) algo_id = pick_for(h, n_out, tokens, k);
     if (algo_id < 0 || !algo_feasible(algo_id, n_out, tokens, k, h->scratch))
@@ -443,6 +456,7 @@ int w4a16_gemm_sequence(w4a16_handle* h, const w4a16_gemm_desc* gemms, int count
         if (chk > 0 && tokens != 0) return fail(W4A16_EARG, "GEMM %d of the sequence is empty", i);
     }
     if (tokens == 0 || count == 0) return W4A16_OK;
+    if (int rc = check_device(h)) return rc;
     if (!(flags & W4A16_SEQ_PERSISTENT) || tokens > 16 || count == 1) {
         // one launch per GEMM; stream order gives the dependencies
         for (int i = 0; i < count; ++i) {
@@ -470,6 +484,7 @@ int w4a16_gemm_sequence(w4a16_handle* h, const w4a16_gemm_desc* gemms, int count
 int w4a16_sequence_status(w4a16_handle* h, void* stream)
 {
     if (!h) return fail(W4A16_EARG, "null handle");
+    if (int rc = check_device(h)) return rc;
     hipError_t e = hipStreamSynchronize((hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "w4a16_sequence_status");
     int word = 0;
@@ -509,6 +524,7 @@ int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const 
     if (chk < 0) return chk;
     if (!metrics || capacity <= 0) return fail(W4A16_EARG, "no room for metrics");
     if (chk > 0) return 0;
+    if (int rc = check_device(h)) return rc;
     constexpr int kWarmup = 10, kMeasure = 100;  // gemm_s4_f16.cu:258-259
     hipStream_t   st   = (hipStream_t)stream;
     bool          have = false;
@@ -694,6 +710,7 @@ int w4a16_probe_read(w4a16_handle* h, const void* src, size_t bytes, void* strea
     // the sink (one word per workgroup, practically never written) is the unused tail of the barrier area
     static_assert(kSyncInts - 64 * 40 >= 8 * 256, "no room for the probe's sink");
     if (h->cus > 256) return fail(W4A16_ESHAPE, "probe_read: more than 256 CUs");
+    if (int rc = check_device(h)) return rc;
     const hipError_t e = launch_probe_read(src, bytes, h->sync + 64 * 40, h->cus, (hipStream_t)stream);
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "probe_read");
 }
@@ -702,6 +719,7 @@ int w4a16_probe_barrier(w4a16_handle* h, int iters, int tree, void* stream)
 {
     if (!h) return fail(W4A16_EARG, "null handle");
     if (iters < 1 || iters > (1 << 20)) return fail(W4A16_EARG, "probe_barrier: iters out of range");
+    if (int rc = check_device(h)) return rc;
     const hipError_t e = launch_probe_barrier(h->sync, iters, tree, h->cus, h->spin_ticks, (hipStream_t)stream);
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "probe_barrier");
 }
