@@ -117,21 +117,15 @@ __device__ __forceinline__ float hi_float(uint64_t v) { return __builtin_bit_cas
 // LDS, dequantised weights - are requested and prepared during the previous one.  A 64-token tile
 // has only 4 * NTW MFMAs per k32 chunk, too few to cover the LDS latency; two chunks per sub-step
 // double the cover at the price of a second set of fragment registers.
-// KW = K slices inside the workgroup (1, 2 or 4): the workgroup is KW sets of WAVES waves; set s works
-// through its own share of the workgroup's groups with its own activation buffers, all sets in step
-// (same number of K steps, shared barriers), and the partial tiles are added in LDS at the end, in slice
-// order.  For small tiles on few tokens, where one set per CU cannot hide its own latencies and splitting
-// K across workgroups costs a round trip through memory.
-template<int TTILES, int NTW, int WAVES, int D, int KS, int EPI, int KW = 1>
-__global__ void __launch_bounds__(64 * WAVES * KW)
-    __attribute__((amdgpu_waves_per_eu(
-        KW > 1 ? WAVES * KW / 4 : (TTILES * NTW * KS >= 16 && WAVES == 4 && (TTILES * NTW >= 32 || KS == 2) ? 1 : 2),
-        KW > 1 ? WAVES * KW / 4 : (TTILES * NTW * KS >= 16 && WAVES == 4 && (TTILES * NTW >= 32 || KS == 2) ? 1 : 2))))
+template<int TTILES, int NTW, int WAVES, int D, int KS, int EPI>
+__global__ void __launch_bounds__(64 * WAVES)
+    __attribute__((amdgpu_waves_per_eu(TTILES * NTW * KS >= 16 && WAVES == 4 && (TTILES * NTW >= 32 || KS == 2) ? 1 : 2,
+                                       TTILES * NTW * KS >= 16 && WAVES == 4 && (TTILES * NTW >= 32 || KS == 2) ? 1 : 2)))
 prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const uint16_t* __restrict__ X,
                const uint32_t* __restrict__ Q, const uint16_t* R_, int N, int T, int K, int tiles_t, int tiles_n,
                float* ws, int* cnt)
 {
-    extern __shared__ __attribute__((aligned(16))) uint8_t xs_all[];  // [KW][D][TT][kRowBytes]
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [D][TT][kRowBytes]
     constexpr int TT = 16 * TTILES;
     constexpr int TN = 16 * NTW * WAVES;
     constexpr int XB = 4 * TTILES / WAVES;  // 1 KiB activation blocks (4 token rows) that each wave fetches per group
@@ -140,13 +134,9 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     static_assert(KS == 1 || KS == 2, "a group is four k32 chunks; sub-steps alternate in parity");
     constexpr int kSub = 4 / KS;  // sub-steps per group
 
-    static_assert(KW == 1 || KW == 2 || KW == 4, "K slices inside the workgroup");
-    const int      lane   = threadIdx.x & 63;
-    const int      wave_g = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int      wave   = KW > 1 ? wave_g % WAVES : wave_g;  // position along the features
-    const int      kslice = KW > 1 ? wave_g / WAVES : 0;
-    const int      tid    = KW > 1 ? (int)threadIdx.x - kslice * 64 * WAVES : (int)threadIdx.x;  // within the set
-    uint8_t* const xs     = xs_all + kslice * (D * TT * kRowBytes);
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c    = lane & 15;
     const int b    = lane >> 4;
     const int G    = K / kGroup;
@@ -172,12 +162,10 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     }
     // split K: blockIdx.y takes the quantisation groups [gbeg, gend), dealt in pairs so that only
     // the last split can have an odd number of them
-    // (with K slices inside the workgroup, slice s of workgroup y is share y * KW + s of splits * KW)
     const int splits = gridDim.y;
     const int pairs  = (G + 1) / 2;
-    const int share  = blockIdx.y * KW + kslice, shares = splits * KW;
-    const int gbeg   = min(G, 2 * (int)((int64_t)pairs * share / shares));
-    const int gend   = min(G, 2 * (int)((int64_t)pairs * (share + 1) / shares));
+    const int gbeg   = min(G, 2 * (int)((int64_t)pairs * blockIdx.y / splits));
+    const int gend   = min(G, 2 * (int)((int64_t)pairs * (blockIdx.y + 1) / splits));
     const int T0     = tile_t * TT;
     const int nt0    = (tile_n * TN) / kTileN + wave * NTW;  // first weight tile of this wave
 
@@ -265,15 +253,12 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     half8_t xf[2][KS][TTILES];
     half2_t z1024[2][NTW], z64[2][NTW], sc[2][NTW];
 
-    // live = false (K slices inside the workgroup only): a step past the end of this slice, which the
-    // slice runs because the others still have groups; its weights count as zero
-    auto split = [&](auto P_, uint32_t (&qv)[NTW], bool live) {
+    auto split = [&](auto P_, uint32_t (&qv)[NTW]) {
         constexpr int P = decltype(P_)::value;
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) {
             half_t s;
             split_q(qv[nt], z1024[P][nt], z64[P][nt], s);
-            if constexpr (KW > 1) s = live ? s : (half_t)0.f;
             sc[P][nt] = half2_t{s, s};
         }
     };
@@ -319,36 +304,22 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     // multiple of D is padded with phantom groups in front: their activation tile is zero-filled
     // LDS instead of a load and their weights are those of the first real group, so they add
     // exactly zero.
-    // With K slices inside the workgroup every slice must run the same number of K steps (they share the
-    // barriers): the longest slice's, rounded up to D; there the surplus steps come last, re-read the
-    // slice's last group and multiply it by a scale of zero (see `split`), and nothing is padded in front.
-    int steps = 0;
-    if constexpr (KW > 1) {
-#pragma unroll
-        for (int sl = 0; sl < KW; ++sl) {
-            const int b = min(G, 2 * (int)((int64_t)pairs * (blockIdx.y * KW + sl) / shares));
-            const int e = min(G, 2 * (int)((int64_t)pairs * (blockIdx.y * KW + sl + 1) / shares));
-            steps       = max(steps, (e - b + D - 1) / D * D);
-        }
-    }
-    const int pad    = KW > 1 ? 0 : (D - (gend - gbeg) % D) % D;
+    const int pad    = (D - (gend - gbeg) % D) % D;
     const int gstart = gbeg - pad;
-    const int gstop  = KW > 1 ? gbeg + steps : gend;
     static_for<0, D>([&](auto dc) {
         constexpr int d  = decltype(dc)::value;
         uint8_t* const xd = xs + d * TT * kRowBytes;
-        const int      gd = min(max(gstart + d, gbeg), gend - 1);
-        issue_w(w[d], q[d], gd);
+        issue_w(w[d], q[d], max(gstart + d, gbeg));
         if (gstart + d < gbeg) {
             for (int i = tid; i < TT * 16; i += 64 * WAVES) reinterpret_cast<u32x4_t*>(xd)[i] = u32x4_t{0, 0, 0, 0};
         }
         else {
-            issue_x(xd, gd);
+            issue_x(xd, gstart + d);
         }
     });
     static_for<0, D>([&](auto dc) { wait_stage(I0{}, w[decltype(dc)::value], q[decltype(dc)::value]); });
     __syncthreads();
-    split(I0{}, q[0], true);
+    split(I0{}, q[0]);
     static_for<0, KS>([&](auto kc) {
         read_x(kc, xs);
         dequant(I0{}, kc, w[0]);
@@ -388,7 +359,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
             const uint32_t rbase =
                 (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)(last ? xo : (const uint8_t*)xb);
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (last) split(PN{}, q[SN], g + 1 < gend);
+            if constexpr (last) split(PN{}, q[SN]);
             // one MFMA, then its share of the next sub-step's dequantisation, and so on
             constexpr int kOps = 13 * NTW * KS, kSlots = TTILES * NTW * KS, kReads = TTILES * KS;
             static_for<0, kSlots>([&](auto ic) {
@@ -425,7 +396,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
 
     // Whole multiples of D only (see `pad` above): no K step outside the loop, so the compiler never
     // has a reason to move an accumulator while the loop's MFMAs may still be writing it.
-    for (int g = gstart; g + D - 1 < gstop; g += D) {  // no branch inside: the 4*TTILES*NTW accumulators stay in place
+    for (int g = gstart; g + D - 1 < gend; g += D) {  // no branch inside: the 4*TTILES*NTW accumulators stay in place
         static_for<0, D>([&](auto dc) { step(dc, g + decltype(dc)::value); });
     }
     // no load may still be writing LDS or registers when the wave ends
@@ -469,32 +440,6 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         }
     };
 
-    // ---- K slices inside the workgroup: add them in LDS, in slice order; slice 0 carries the tile on ----
-    const bool lead = kslice == 0;
-    if constexpr (KW > 1) {
-        constexpr int   kTilesW = TTILES * NTW;
-        float4_t* const red     = reinterpret_cast<float4_t*>(xs_all);  // [KW - 1][WAVES][kTilesW][64 lanes]
-        static_assert((KW - 1) * WAVES * kTilesW * 1024 <= KW * D * TT * kRowBytes, "the partial tiles reuse the activation buffers");
-        __syncthreads();  // every wave is done with the activation tiles
-        if (!lead) {
-#pragma unroll
-            for (int tt = 0; tt < TTILES; ++tt)
-#pragma unroll
-                for (int nt = 0; nt < NTW; ++nt)
-                    red[(((kslice - 1) * WAVES + wave) * kTilesW + tt * NTW + nt) * 64 + lane] = acc[tt][nt];
-        }
-        __syncthreads();
-        if (lead) {
-#pragma unroll
-            for (int sl = 1; sl < KW; ++sl)
-#pragma unroll
-                for (int tt = 0; tt < TTILES; ++tt)
-#pragma unroll
-                    for (int nt = 0; nt < NTW; ++nt)
-                        acc[tt][nt] += red[(((sl - 1) * WAVES + wave) * kTilesW + tt * NTW + nt) * 64 + lane];
-        }
-    }
-
     // ---- split K: exchange partial tiles through the workspace ----
     // Each wave writes its accumulators as it holds them (per tile two 512-byte rows, lane l the
     // floats 2l, 2l+1), with agent-scope atomic stores and loads: the L2 caches of the XCDs are not
@@ -510,7 +455,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         int lane_now = lane;
         asm volatile("" : "+v"(lane_now));
         float* const  mine_base = ws + ((int64_t)id * WAVES + wave) * kTiles * 256 + lane_now * 2;
-        if (lead) {
+        {
             float* wp = mine_base + blockIdx.y * per_split;
 #pragma unroll
             for (int tt = 0; tt < TTILES; ++tt)
@@ -524,8 +469,8 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         }
         __builtin_amdgcn_s_waitcnt(0);  // all of this wave's stores are complete
         __syncthreads();                // ... and every wave is done with the activation tiles in LDS
-        int* const last_flag = reinterpret_cast<int*>(xs_all);
-        if (threadIdx.x == 0) {
+        int* const last_flag = reinterpret_cast<int*>(xs);
+        if (tid == 0) {
             int* const cp   = cnt + id;
             const int  old  = __hip_atomic_fetch_add(cp, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const bool last = old == splits - 1;
@@ -533,7 +478,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
             *last_flag = last;
         }
         __syncthreads();
-        if (!*last_flag || !lead) return;
+        if (!*last_flag) return;
 #pragma unroll
         for (int tt = 0; tt < TTILES; ++tt)
 #pragma unroll
@@ -563,7 +508,6 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     }
 
     // ---- epilogue: lane (c, b) of tile (tt, nt) holds token T0 + 16 tt + c, features n .. n+3 ----
-    if (!lead) return;
 #pragma unroll
     for (int tt = 0; tt < TTILES; ++tt)
 #pragma unroll
@@ -574,11 +518,9 @@ struct Variant {
     int ttiles, ntw, waves, depth, chunks;
     // Measured on MI355X (K = 2048 against 6144, cold weights): microseconds per K step for the whole
     // grid at 1, 2, 3, 4 and 8 workgroups per CU.  Tiles that fill a CU by themselves go in rounds.
-    // (The two-chunk rows are the one-chunk measurements x 0.96, the ratio seen on Llama-7B shapes; the rows with
-    // K slices inside the workgroup are fitted to Llama-7B qkv, o and gate_up at 64 to 256 tokens, one round = one row.)
+    // (The two-chunk rows are the one-chunk measurements x 0.96, the ratio seen on Llama-7B shapes.)
     bool  one_per_cu;
     float step_us[5];
-    int   kw = 1;  // K slices inside the workgroup (sets of `waves` waves)
 };
 // (a 256 x 256 tile does not fit the register file without spilling, and spill stores would
 // break the counted waits: stores and loads complete out of order with each other)
@@ -590,25 +532,21 @@ constexpr Variant kVariants[] = {
     {4, 1, 4, 4, 2, false, {0.425f, 0.673f, 1.000f, 1.340f, 2.833f}},   //  64 x 64, two chunks per sub-step
     {4, 1, 8, 4, 2, true, {0.553f, 1.209f, 1.906f, 2.609f, 5.351f}},    //  64 x 128, eight waves, two chunks per sub-step
     {4, 2, 8, 4, 1, true, {1.034f, 2.290f, 3.605f, 4.644f, 8.583f}},    //  64 x 256, eight waves
-    // two K slices inside the workgroup (per K step of the workgroup, i.e. two groups).  Four slices of four
-    // waves would need the kernel in 128 registers per wave, where the allocator starts parking values in AGPRs.
-    {4, 1, 4, 4, 2, true, {0.830f, 1.660f, 2.490f, 3.320f, 6.640f}, 2},   //  64 x 64, 4 x 2 waves
-    {4, 2, 4, 4, 1, true, {1.420f, 2.840f, 4.260f, 5.680f, 11.360f}, 2},  //  64 x 128, 4 x 2 waves
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
-template<int TTILES, int NTW, int WAVES, int D, int KS, int KW = 1>
+template<int TTILES, int NTW, int WAVES, int D, int KS>
 hipError_t launch_v(int splits, const GemmArgs& a, const Scratch& sc, hipStream_t st)
 {
     constexpr int TT = 16 * TTILES, TN = 16 * NTW * WAVES;
     const int     tiles_t = (a.T + TT - 1) / TT;
     const int     tiles_n = a.N / TN;
-    const size_t  lds     = (size_t)KW * D * TT * kRowBytes;
-    const dim3    grid(tiles_t * tiles_n, splits), block(64 * WAVES * KW);
+    const size_t  lds     = (size_t)D * TT * kRowBytes;
+    const dim3    grid(tiles_t * tiles_n, splits), block(64 * WAVES);
     const u32x4_t* A4 = reinterpret_cast<const u32x4_t*>(a.A);
 #define W4A16_LAUNCH(EPI)                                                                                              \
     do {                                                                                                               \
-        auto                         kfn = prefill_kernel<TTILES, NTW, WAVES, D, KS, EPI, KW>;                         \
+        auto                         kfn = prefill_kernel<TTILES, NTW, WAVES, D, KS, EPI>;                             \
         static std::atomic<uint64_t> raised{0}; /* per instantiation, one bit per device */                            \
         const hipError_t             e = raise_lds_limit(reinterpret_cast<const void*>(kfn), (int)lds, raised);        \
         if (e != hipSuccess) return e;                                                                                 \
@@ -652,10 +590,9 @@ bool prefill_feasible(int v, int splits, int N, int T, int K, size_t ws_bytes, i
     // per-thread offsets into X and into one group of A are 32-bit
     if ((int64_t)T * K * 2 >= (1ll << 32) || (int64_t)N * 64 >= (1ll << 32)) return false;
     const int64_t grid = (int64_t)(N / tn) * ((T + tt - 1) / tt);
-    if (K / kGroup < 2 * kVariants[v].kw) return false;  // at least two groups per K slice
     if (splits > 1) {
         // at least two groups per split; partial tiles and counters must fit the handle's scratch
-        if (K / kGroup < 2 * splits * kVariants[v].kw || splits > 65535) return false;
+        if (K / kGroup < 2 * splits || splits > 65535) return false;
         if (grid * splits * tn * tt * 4 > (int64_t)ws_bytes || grid > cnt_len) return false;
     }
     return grid * splits < (1ll << 31);
@@ -678,9 +615,7 @@ hipError_t prefill_launch(int v, int splits, const GemmArgs& a, const Scratch& s
         case 3: return launch_v<4, 2, 4, 4, 1>(splits, a, sc, st);
         case 4: return launch_v<4, 1, 4, 4, 2>(splits, a, sc, st);
         case 5: return launch_v<4, 1, 8, 4, 2>(splits, a, sc, st);
-        case 6: return launch_v<4, 2, 8, 4, 1>(splits, a, sc, st);
-        case 7: return launch_v<4, 1, 4, 4, 2, 2>(splits, a, sc, st);
-        default: return launch_v<4, 2, 4, 4, 1, 2>(splits, a, sc, st);
+        default: return launch_v<4, 2, 8, 4, 1>(splits, a, sc, st);
     }
 }
 
@@ -710,7 +645,7 @@ double prefill_estimate_us(int v, int splits, int N, int T, int K)
     if (var.one_per_cu && load < 1.0) step *= 0.7 + 0.3 * load;
     if (!var.one_per_cu && var.ttiles == 4 && load > 2.0) step *= 1.25;
     const int groups = K / kGroup;
-    int       steps  = (groups + splits * var.kw - 1) / (splits * var.kw);
+    int       steps  = (groups + splits - 1) / splits;
     steps            = (steps + var.depth - 1) / var.depth * var.depth;  // phantom groups
     double us = 3.0 + steps * step;
     if (splits > 1) {
