@@ -24,6 +24,7 @@ import argparse
 import json
 import os
 import sys
+import threading
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -80,6 +81,24 @@ def make_weights(tm, torch, gen, name, K, N):
     return A, Q
 
 
+def read_power_and_clocks():
+    """Socket power and per-XCD engine clocks from `amd-smi metric --power --clock` (a sensor read; a child
+    process, so that nothing is started in place of this one)."""
+    import re
+    import subprocess
+    tool = "amd-smi metric --power --clock"
+    try:
+        out = subprocess.run(tool.split(), capture_output=True, text=True, timeout=30).stdout
+    except (OSError, subprocess.SubprocessError) as e:
+        return {"tool": tool, "error": str(e)[:200]}
+    power = re.search(r"SOCKET_POWER:\s*(\d+)\s*W", out)
+    clocks = [int(m) for m in re.findall(r"GFX_\d+:\s*\n\s*CLK:\s*(\d+)\s*MHz", out)]
+    if not power and not clocks:
+        return {"tool": tool, "error": "no power or clock figures in the tool's output"}
+    return {"tool": tool, "socket_power_W": int(power.group(1)) if power else None, "gfx_clk_MHz": clocks,
+            "mean_gfx_clk_MHz": round(sum(clocks) / len(clocks), 1) if clocks else None}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -95,6 +114,8 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-per-shape", action="store_true")
     ap.add_argument("--no-70b", action="store_true")
+    ap.add_argument("--no-sustained", action="store_true", help="skip the power / clock reading under a sustained prefill load")
+    ap.add_argument("--sustained-seconds", type=float, default=4.0)
     ap.add_argument("--seconds", type=float, default=8.0, help="duration of the sustain-* probes")
     ap.add_argument("--probe", choices=["decode", "prefill", "decode-o", "sequence-trace", "sustain-prefill",
                                         "sustain-decode", "sustain-dense"],
@@ -317,6 +338,36 @@ def main():
                                 "unit": "TFLOP/s", "frac": dom["frac"],
                                 "traffic": TRAFFIC_PREFILL_GATE_UP if dom["shape"] == "gate_up" else None,
                                 "kernel": "prefill_kernel, %s, T=2048" % dom["shape"]}}
+
+        # The same kernel kept running for a few seconds, with the socket power and the engine clocks read beside
+        # it: the 2.5 PFLOP/s peak is quoted at 2.4 GHz, and under a sustained matrix load the GPU sits at its
+        # power limit and clocks lower.
+        if not args.no_sustained:
+            name = dom["shape"]
+            r = make_runner([[(name, c, PREFILL_T) for c in range(4)]])
+            reps = max(1, int(args.sustained_seconds * 1e3 / (dom["ms"] * 4)))
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            sensors = {}
+            # (a thread: enqueueing thousands of replays may block this one until most of them have run)
+            reader = threading.Thread(target=lambda: (time.sleep(min(1.5, args.sustained_seconds / 3)),
+                                                      sensors.update(read_power_and_clocks())))
+            torch.cuda.synchronize()
+            reader.start()
+            e0.record(stream)
+            with torch.cuda.stream(stream):
+                for _ in range(reps):
+                    r[0]()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            reader.join()
+            fl = flops(PREFILL_T, *shape[name][:2])
+            sensors.update(kernel="prefill_kernel, %s, T=2048" % name, seconds=round(e0.elapsed_time(e1) / 1e3, 2),
+                           TFLOPs=round(4 * reps * fl / e0.elapsed_time(e1) / 1e9, 1))
+            if sensors.get("mean_gfx_clk_MHz"):
+                at_clock = MFMA_PEAK_TFLOPS * sensors["mean_gfx_clk_MHz"] / 2400.0
+                sensors.update(mfma_peak_at_that_clock_TFLOPs=round(at_clock, 1),
+                               frac_of_peak_at_that_clock=round(sensors["TFLOPs"] / at_clock, 4))
+            prefill["under_sustained_load"] = sensors
 
     # ---- the full 32-layer GEMM sequence of one decode step at M = 8 (every layer its own weights) ----
     # as one launch per GEMM, and through w4a16_gemm_sequence as persistent launches (32 GEMMs each, every GEMM
