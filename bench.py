@@ -12,7 +12,9 @@ algorithmic bytes of all launches / elapsed time.
 Also in the same JSON line: roofline objects for the dominant decode kernel (gate_up) and for the
 one furthest below its roofline (o), per-shape tables for Llama-2-7B and Llama-2-70B (decode:
 GB/s; T = 2048: TFLOP/s), the 32-layer decode step at M = 8 as one launch per GEMM and as
-persistent launches, what plain library kernels reach on this GPU (streaming reads of 8 / 45 /
+persistent launches, the socket power and engine clocks read while the prefill kernel runs for
+four seconds (the part sits at its power limit and well below the 2.4 GHz of its quoted peak), what
+plain library kernels reach on this GPU (streaming reads of 8 / 45 /
 512 MiB, a device copy, a dense fp16 GEMM), and the CPU baseline (the oracle: unpack,
 dequantise, torch fp32 matmul) timed on the host cores on bounded samples.
 
