@@ -119,13 +119,11 @@ def main():
     ap.add_argument("--no-sustained", action="store_true", help="skip the power / clock reading under a sustained prefill load")
     ap.add_argument("--sustained-seconds", type=float, default=4.0)
     ap.add_argument("--seconds", type=float, default=8.0, help="duration of the sustain-* probes")
-    ap.add_argument("--probe", choices=["decode", "prefill", "decode-o", "sequence-trace", "sustain-prefill",
+    ap.add_argument("--probe", choices=["decode", "prefill", "decode-o", "sustain-prefill",
                                         "sustain-decode", "sustain-dense"],
                     help="decode / prefill / decode-o: run only the named kernel (gate_up decode / gate_up at T=2048 / o "
                          "decode) plus a plain 256 MiB elementwise kernel, eagerly, for `rocprofv3 --pmc` (no JSON line).  "
-                         "sequence-trace: print the in-kernel time stamps of the persistent sequence kernel over Llama-2-7B "
-                         "layers at T=8 (needs W4A16_LIB=lmdeploy_amd/lib/libw4a16_trace.so from "
-                         "`python -m lmdeploy_amd.build --trace`).  sustain-prefill / sustain-decode / sustain-dense: "
+                         "sustain-prefill / sustain-decode / sustain-dense: "
                          "keep launching gate_up (T=2048 / T=8 / torch.matmul fp16 at T=2048) for --seconds and print the "
                          "rate once a second, so that the engine clock under that load can be read beside it "
                          "(`rocm-smi --showclocks`)")
@@ -138,10 +136,6 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
-    trace = None
-    if args.probe == "sequence-trace":   # the tracing build reads the buffer's address from the environment at launch
-        trace = torch.zeros(4 * 256 * 8, dtype=torch.int64, device="cuda")
-        os.environ["W4A16_TRACE_PTR"] = "%x" % trace.data_ptr()
     import lmdeploy_amd.turbomind as tm
 
     torch.cuda.set_device(0)
@@ -155,9 +149,7 @@ def main():
     for name, K, N, epi in LAYER_7B:
         per_copy = K * N // 2 + (K // GROUP) * N * 4
         n = max(len(DECODE_T) * n_sets, N_LAYERS, int(args.cold_gib * 2 ** 30 / per_copy) + 1)
-        if args.probe == "sequence-trace":
-            n = 16
-        elif args.probe:
+        if args.probe:
             n = max(8, int(args.cold_gib * 2 ** 30 / per_copy) + 1) if name in ("gate_up", "o") else 1
         weights[name] = [make_weights(tm, torch, gen, name, K, N) for _ in range(n)]
     Tmax = max(max(DECODE_T), PREFILL_T)
@@ -200,34 +192,6 @@ def main():
             e1.record(stream)
             torch.cuda.synchronize()
         return e0.elapsed_time(e1)   # ms
-
-    if args.probe == "sequence-trace":
-        T, L = 8, 16
-        descs = []
-        for layer in range(L):
-            for name, K, N, epi in LAYER_7B:
-                A, Q = weights[name][layer]
-                descs.append((out[name], A, X[K], Q, N, K, epi, Res if epi == 2 else None, bool(descs)))
-        for rep in range(3):
-            for i in range(0, len(descs), 32):
-                gemm.sequence(descs[i:i + 32], T, persistent=True)
-            gemm.sequence_status()
-        t = trace.cpu().view(4, 256, 8).numpy()
-        if not t.any():
-            print("no time stamps: W4A16_LIB must name the tracing build (python -m lmdeploy_amd.build --trace)")
-            return
-        print("persistent sequence kernel, Llama-2-7B layers at T=8, second launch of 32 GEMMs; microseconds after the moment the "
-              "GEMM's inputs were ready (device-wide barrier passed), lane 0 of the named wave")
-        print("columns: first = first two groups multiplied | loop = K loop done | epi = sums reduced, outputs stored | "
-              "drained = stores written through | next = the next GEMM's inputs ready (its first weights were requested before the barrier)")
-        for who, label in enumerate(["workgroup 0 wave 0", "workgroup 0 wave 7", "workgroup 131 wave 0", "workgroup 131 wave 7"]):
-            print(label)
-            for u in range(8, 16):
-                r, nxt = t[who, u], t[who, u + 1]
-                f = lambda v: (v - r[0]) / 100.0
-                print("  %-8s first %5.2f | loop %5.2f | epi %5.2f | drained %5.2f | next %5.2f" % (
-                    LAYER_7B[u % 4][0], f(r[1]), f(r[2]), f(r[3]), f(nxt[4]), f(nxt[0])))
-        return
 
     if args.probe and args.probe.startswith("sustain-"):
         K, N, _ = shape["gate_up"]

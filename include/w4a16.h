@@ -138,15 +138,19 @@ typedef struct w4a16_gemm_desc {
  * kept for callers for whom launches are dearer than that (no graphs, a busy host thread).
  * The persistent launch needs its workgroups resident all at once, which holds when nothing else
  * occupies the GPU's CUs for long; its barrier waits are bounded (w4a16_set_barrier_timeout, default
- * 2 s): a workgroup that gives up sets an error word in the handle, and every workgroup still
- * finishes.  Nothing is allocated and nothing synchronises, so the call can be captured in a HIP
+ * 50 ms): a workgroup that gives up sets an error word in the handle, and every workgroup still
+ * finishes.  The error word is sticky: until w4a16_sequence_status has been called, every later
+ * persistent launch on this handle passes its barriers without waiting, so its outputs are
+ * undefined too.  A caller that replays a captured persistent launch must therefore poll
+ * w4a16_sequence_status (between replays; it synchronises the stream).  Nothing is allocated and nothing synchronises, so the call can be captured in a HIP
  * graph (for T > 16, and for matrices that split K, after one call outside capture: see w4a16_create). */
 #define W4A16_SEQ_PERSISTENT 1
 int w4a16_gemm_sequence(w4a16_handle* h, const w4a16_gemm_desc* gemms, int count, int tokens, int group_size,
                         int flags, void* stream);
 
 /* Synchronises `stream` and reports whether a barrier of an earlier w4a16_gemm_sequence on this handle
- * gave up: W4A16_OK, or W4A16_ETIMEOUT (once; the handle is usable again afterwards). */
+ * gave up: W4A16_OK, or W4A16_ETIMEOUT (once; the barrier state is then cleared on `stream` and the handle
+ * is usable again).  Outputs of every persistent launch between the timeout and this call are undefined. */
 int w4a16_sequence_status(w4a16_handle* h, void* stream);
 
 /* Time limit of one barrier wait of w4a16_gemm_sequence, 0 .. 3600 seconds. */
@@ -251,17 +255,6 @@ int w4a16_dequantize_repacked(void* W, const uint32_t* A, const void* Q, int m, 
  * convert_s4_k_m8, i.e. a `.qweight` file written by deploy.py:142-146) to the gfx950
  * layout.  Q needs no conversion.  m % 32 == 0, k % 128 == 0. */
 int w4a16_from_reference_layout(uint32_t* A_dst, const uint32_t* A_ref, int m, int k, void* stream);
-
-/* Measurement aid (no counterpart in the reference): a plain streaming read of `bytes` at `src`,
- * launched like the decode kernels.  Its time on a buffer of a matrix's size is the ceiling that a
- * launch, the first trip to HBM and the streaming itself set for a GEMM that reads the matrix once. */
-int w4a16_probe_read(w4a16_handle* h, const void* src, size_t bytes, void* stream);
-
-/* Measurement aid (no counterpart in the reference): one persistent launch of one workgroup per CU that
- * crosses `iters` device-wide barriers of w4a16_gemm_sequence and does nothing else; time it with
- * events and divide.  tree = 1: the two-level counter tree that the sequence kernel uses; tree = 0: every
- * workgroup arrives on one counter. */
-int w4a16_probe_barrier(w4a16_handle* h, int iters, int tree, void* stream);
 
 const char* w4a16_last_error(void);
 const char* w4a16_version(void);

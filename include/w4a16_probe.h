@@ -1,0 +1,30 @@
+/*
+ * Measurement aids of libw4a16.so.  Nothing here belongs to the GEMM path or has a counterpart in
+ * the reference: these entry points exist so that a benchmark can time what the machine gives a
+ * kernel that does nothing but read, or nothing but synchronise, launched the way the GEMM
+ * kernels are.  Conventions (pointers, streams, return codes) are those of w4a16.h.
+ */
+#ifndef W4A16_PROBE_H_
+#define W4A16_PROBE_H_
+
+#include "w4a16.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Measurement aid (no counterpart in the reference): a plain streaming read of `bytes` at `src`,
+ * launched like the decode kernels.  Its time on a buffer of a matrix's size is the ceiling that a
+ * launch, the first trip to HBM and the streaming itself set for a GEMM that reads the matrix once. */
+int w4a16_probe_read(w4a16_handle* h, const void* src, size_t bytes, void* stream);
+
+/* Measurement aid (no counterpart in the reference): one persistent launch of one workgroup per CU that
+ * crosses `iters` device-wide barriers of w4a16_gemm_sequence and does nothing else; time it with
+ * events and divide.  tree = 1: the two-level counter tree that the sequence kernel uses; tree = 0: every
+ * workgroup arrives on one counter. */
+int w4a16_probe_barrier(w4a16_handle* h, int iters, int tree, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* W4A16_PROBE_H_ */

@@ -113,26 +113,6 @@ def build_library(verbose: bool = True) -> str:
     return LIB_PATH
 
 
-def build_trace_library(verbose: bool = True) -> str:
-    """A variant of the library whose persistent sequence kernel records in-kernel time stamps
-    (-DW4A16_TRACE, see csrc/gemm_sequence.hip), as lib/libw4a16_trace.so.  It reuses the objects of
-    `build_library`; select it with W4A16_LIB and run `bench.py --probe sequence-trace`."""
-    obj_dir = os.path.join(HERE, "build")
-    obj = os.path.join(obj_dir, "gemm_sequence_trace.o")
-    r = subprocess.run([_hipcc(), *HIP_FLAGS, "-DW4A16_TRACE", "-c", os.path.join(CSRC, "gemm_sequence.hip"), "-o", obj],
-                       capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("hipcc failed for the tracing build:\n%s\n%s" % (r.stdout, r.stderr))
-    objs = [os.path.join(obj_dir, os.path.splitext(s)[0] + ".o") for s in SOURCES if s != "gemm_sequence.hip"] + [obj]
-    out = os.path.join(LIB_DIR, "libw4a16_trace.so")
-    r = subprocess.run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *objs], capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
-    if verbose:
-        print("built", out)
-    return out
-
-
 def check_headers(verbose: bool = True) -> str:
     """Compiles and links tests/cpp/llama_linear_dropin.cpp against the C++ front-end headers and
     the library: the proof that a LlamaLinear-shaped caller builds against them."""
@@ -155,6 +135,4 @@ def check_headers(verbose: bool = True) -> str:
 if __name__ == "__main__":
     build_library()
     check_headers()
-    if "--trace" in sys.argv[1:]:
-        build_trace_library()
     sys.exit(0)

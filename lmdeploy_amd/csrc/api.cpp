@@ -1,6 +1,7 @@
 // The C ABI of libw4a16.so: argument validation, kernel selection, timing and error
 // reporting.  No kernel code lives here.
 #include "../../include/w4a16.h"
+#include "../../include/w4a16_probe.h"
 #include "w4a16_internal.h"
 
 #include <algorithm>
@@ -322,7 +323,7 @@ int w4a16_create(w4a16_handle** out)
     int khz = 0;
     if (e == hipSuccess) e = hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, h->device);
     h->clock_khz  = khz > 0 ? khz : 100000;
-    h->spin_ticks = 2000 * h->clock_khz;  // two seconds
+    h->spin_ticks = 50 * h->clock_khz;  // 50 ms: a serving loop must not stall for longer than that
     if (e == hipSuccess) e = hipDeviceSynchronize();
     // a library set-up call on this device: also the moment to look up the static scratch array's address
     Scratch st{};
@@ -491,7 +492,9 @@ int w4a16_sequence_status(w4a16_handle* h, void* stream)
     e = hipMemcpy(&word, h->sync + sequence_error_index(), sizeof(int), hipMemcpyDeviceToHost);
     if (e != hipSuccess) return hip_fail(e, "w4a16_sequence_status");
     if (word == 0) return W4A16_OK;
-    e = hipMemset(h->sync, 0, kSyncInts * sizeof(int));  // the launch that gave up may have left counters behind
+    // the launch that gave up may have left counters behind; cleared in stream order, then waited for
+    e = hipMemsetAsync(h->sync, 0, kSyncInts * sizeof(int), (hipStream_t)stream);
+    if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "w4a16_sequence_status");
     return fail(W4A16_ETIMEOUT, "a workgroup of w4a16_gemm_sequence gave up waiting at a device-wide barrier: the "
                                 "grid was not resident all at once; the outputs of that launch are undefined");

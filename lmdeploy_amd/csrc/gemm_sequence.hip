@@ -107,7 +107,6 @@ __global__ void __launch_bounds__(64 * kWaves) sequence_kernel(const SeqArgs a)
     const int strips = gridDim.x;
 
     int barrier_no = 0;
-    [[maybe_unused]] int trace_unit = 0;
     for (int i = 0; i < a.count; ++i) {
         const SeqGemm& g      = a.g[i];
         const int      NT     = g.N / kTileN;
@@ -115,9 +114,8 @@ __global__ void __launch_bounds__(64 * kWaves) sequence_kernel(const SeqArgs a)
         for (int pass = 0; pass < passes; ++pass) {
             // this wave's output stores of the previous unit are complete (written through to memory)
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            W4A16_STAMP(4);
             const Strip st = strip_of(NT, strips, passes, pass, bx);
-            StripParams p{g.C, g.A, g.X, g.Q, g.R, g.N, a.T, g.K, 0, 0, trace_unit, g.epilogue};
+            StripParams p{g.C, g.A, g.X, g.Q, g.R, g.N, a.T, g.K, 0, 0, g.epilogue};
             // called by every wave once its first weight loads are on their way
             auto ready = [&]() {
                 workgroup_barrier();  // every wave has drained its stores and is done with the sums in LDS
@@ -126,7 +124,6 @@ __global__ void __launch_bounds__(64 * kWaves) sequence_kernel(const SeqArgs a)
                     ++barrier_no;
                     workgroup_barrier();
                 }
-                W4A16_STAMP(0);
             };
             switch (st.width) {
                 case 1: strip_body<1, TP, kEpiRuntime, true>(p, st.col0, smem, ready); break;
@@ -139,8 +136,6 @@ __global__ void __launch_bounds__(64 * kWaves) sequence_kernel(const SeqArgs a)
                 case 8: strip_body<8, TP, kEpiRuntime, true>(p, st.col0, smem, ready); break;
                 default: ready(); break;  // fewer column tiles than workgroups: nothing to compute in this one
             }
-            W4A16_STAMP(3);
-            ++trace_unit;
         }
     }
     // the last workgroup to leave finds every other one past its last wait: it puts the counters back to zero
@@ -217,12 +212,6 @@ int sequence_error_index()
 hipError_t sequence_launch(const SeqGemm* g, int count, int T, int* sync, int cus, long long spin_ticks, hipStream_t st)
 {
     if (!sequence_feasible(g, count, T) || !sync || cus < 1) return hipErrorInvalidValue;
-#ifdef W4A16_TRACE
-    if (const char* env = getenv("W4A16_TRACE_PTR")) {
-        long long* ptr = (long long*)strtoull(env, nullptr, 16);
-        (void)hipMemcpyToSymbol(HIP_SYMBOL(g_trace), &ptr, sizeof(ptr));
-    }
-#endif
     SeqArgs a{};
     for (int i = 0; i < count; ++i) a.g[i] = g[i];
     a.count      = count;

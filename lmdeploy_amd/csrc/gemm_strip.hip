@@ -139,7 +139,7 @@ hipError_t strip_launch(int per_cu, int block_t, const GemmArgs& a, hipStream_t 
     const int   tp = block_t == 32 ? 32 : (a.T <= 4 ? 4 : (a.T <= 8 ? 8 : 16));
     const int   h  = tp > 16 ? tp / 16 : 1;
     StripParams p{a.C, reinterpret_cast<const u32x4_t*>(a.A), a.X, a.Q, a.R, a.N, a.T, a.K, pl.base, pl.rem,
-                  0, a.epilogue};
+                  a.epilogue};
     const dim3   grid(pl.strips, (a.T + block_t - 1) / block_t);
     // per wave: the sums of its strip, over its activation patch(es) - two for 32 tokens, which arrive straight from memory
     const size_t lds = (size_t)kWaves * std::max(pl.rmax * h * 1024, tp * 256 * (tp >= kDmaTokens ? 2 : 1));

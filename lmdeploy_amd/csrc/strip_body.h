@@ -24,10 +24,7 @@ constexpr int kWaves   = 8;  // = K slices per workgroup
 constexpr int kMaxR    = 8;  // column tiles per strip
 constexpr int kMaxR32  = 8;  // ... with 32 tokens per workgroup
 constexpr int kNumCU   = 256;
-#ifndef W4A16_DMA_TOKENS
-#define W4A16_DMA_TOKENS 32
-#endif
-constexpr int kDmaTokens = W4A16_DMA_TOKENS;  // token block from which the activations go straight to LDS
+constexpr int kDmaTokens = 32;  // token block from which the activations go straight to LDS
 
 struct StripParams {
     uint16_t*       C;
@@ -38,28 +35,10 @@ struct StripParams {
     int             N, T, K;
     int             base;  // column tiles of a narrow strip
     int             rem;   // the first `rem` strips have base + 1
-    int             tag;   // not read by the kernels: the tracing build files its time stamps under this number
     int             epilogue;  // read by kernels whose epilogue is chosen at run time (EPI == kEpiRuntime)
 };
 
 constexpr int kEpiRuntime = 3;  // template value: take the epilogue from StripParams
-
-// Optional in-kernel time stamps (build with -DW4A16_TRACE; see gemm_sequence.hip): slot `s` of unit
-// `u`, recorded by lane 0 of waves 0 and 7 of two workgroups.
-#ifdef W4A16_TRACE
-static __device__ long long* g_trace;
-#define W4A16_STAMP(slot)                                                                                              \
-    do {                                                                                                               \
-        if (g_trace && (threadIdx.x & 63) == 0 && ((threadIdx.x >> 6) == 0 || (threadIdx.x >> 6) == 7) &&              \
-            (blockIdx.x == 0 || blockIdx.x == 131))                                                                    \
-            g_trace[(((blockIdx.x ? 1 : 0) * 2 + ((threadIdx.x >> 6) ? 1 : 0)) * 256 + trace_unit) * 8 + (slot)] =    \
-                wall_clock64();                                                                                        \
-    } while (0)
-#else
-#define W4A16_STAMP(slot)                                                                                              \
-    do {                                                                                                               \
-    } while (0)
-#endif
 
 // Loads of the software pipeline: issued from inline assembly, in place ("+v"), with a scalar
 // base, a per-lane 32-bit offset and an immediate, and waited for by count (the compiler would
@@ -172,7 +151,6 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     // H row blocks of 16 tokens share every unpacked weight (H = 2 for the 32-token variant)
     constexpr int H  = TP > 16 ? TP / 16 : 1;
     const int     t0 = SEQ ? 0 : blockIdx.y * (16 * H);
-    [[maybe_unused]] const int trace_unit = p.tag;
     const int     Tl = min(16 * H, T - t0);
 
     // this wave's groups: wave, wave + 8, wave + 16, ...  Interleaved rather than blocked, so that
@@ -400,9 +378,7 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
             constexpr int d = decltype(dc)::value;
             step(dc, i + d < cnt, g0 + (i + d + D) * kStep, i + d + D < cnt);
         });
-        if (i == 0) W4A16_STAMP(1);
     }
-    W4A16_STAMP(2);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the masked refills of the last trip
 
     // ---- add the eight slices in LDS, in slice order ----

@@ -1,5 +1,5 @@
-"""CPU-side checks of the C ABI: the library loads, exports every symbol that include/w4a16.h
-declares, and rejects bad arguments with the documented codes before touching a GPU.
+"""CPU-side checks of the C ABI: the library loads, exports every symbol that include/*.h
+declare, and rejects bad arguments with the documented codes before touching a GPU.
 (No compute call is made here.)"""
 import ctypes
 import os
@@ -8,7 +8,7 @@ import re
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "w4a16.h")
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("w4a16.h", "w4a16_probe.h")]
 
 
 @pytest.fixture(scope="module")
@@ -18,7 +18,7 @@ def L():
 
 
 def declared_symbols():
-    text = open(HEADER).read()
+    text = "".join(open(h).read() for h in HEADERS)
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(w4a16_[a-z0-9_]+)\s*\(", text)))
 
