@@ -18,6 +18,13 @@ extern "C" {
  * launch, the first trip to HBM and the streaming itself set for a GEMM that reads the matrix once. */
 int w4a16_probe_read(w4a16_handle* h, const void* src, size_t bytes, void* stream);
 
+/* The same read with the load pipeline of the GEMM kernels: every lane keeps `in_flight` (2, 4, 8 or 16)
+ * 16-byte loads in flight, issued in place and waited for by count, `wg_per_cu` (1, 2 or 4) workgroups of
+ * eight waves per CU; hint 0 = plain loads, 1 = non-temporal, 2 = system scope.  `bytes` is rounded down
+ * to a multiple of 1024.  For sweeping what the memory system gives a kernel that only reads. */
+int w4a16_probe_stream(w4a16_handle* h, const void* src, size_t bytes, int wg_per_cu, int in_flight, int hint,
+                       void* stream);
+
 /* Measurement aid (no counterpart in the reference): one persistent launch of one workgroup per CU that
  * crosses `iters` device-wide barriers of w4a16_gemm_sequence and does nothing else; time it with
  * events and divide.  tree = 1: the two-level counter tree that the sequence kernel uses; tree = 0: every

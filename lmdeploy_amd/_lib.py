@@ -65,6 +65,7 @@ SIGNATURES = {
     "w4a16_dequantize_repacked": (c_int, [c_void_p] * 3 + [c_int] * 3 + [c_void_p]),
     "w4a16_from_reference_layout": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "w4a16_probe_read": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "w4a16_probe_stream": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_void_p]),
     "w4a16_probe_barrier": (c_int, [c_void_p, c_int, c_int, c_void_p]),
     "w4a16_last_error": (c_char_p, []),
     "w4a16_version": (c_char_p, []),

@@ -76,7 +76,8 @@ std::vector<Algo> build_table()
         t.push_back(Algo{0, 128, 16, 2, 0, DecodeConfig{1, 8, 2, 4, fill}});
     }
     // strips of column tiles over the whole of K, 1 or 2 per CU
-    for (int per_cu : {1, 2}) t.push_back(Algo{2, 0, 16, 8, per_cu, DecodeConfig{}});
+    // (3: one workgroup per CU that walks several strips in turn, for matrices wider than 8 x 256 column tiles)
+    for (int per_cu : {1, 2, 3}) t.push_back(Algo{2, 0, 16, 8, per_cu, DecodeConfig{}});
     // the same with 32 tokens per workgroup (17 tokens and more): half the passes over the weights
     for (int per_cu : {1, 2}) t.push_back(Algo{2, 0, 32, 8, per_cu, DecodeConfig{}});
     for (int v = 0; v < prefill_variants(); ++v) {
@@ -187,8 +188,10 @@ int algo_pick(int N, int T, int K, const Scratch& lim)
     // Above 16 tokens every workgroup re-reads the weights once per 16-token block, and narrow
     // matrices are better off splitting K across workgroups (column-block kernel with `fill`).
     if (N / 16 >= 128 && (T <= 16 || N / 16 >= 512)) {
+        // (3 = one workgroup per CU taking several strips in turn: only feasible, and then measured 2 - 6 % ahead, for
+        // matrices too wide for one strip per CU, such as the 57344 columns of Llama-2-70B's gate_up)
         const int want = (N / 16 >= 1024 && T <= 8) ? 2 : 1;
-        for (int per_cu : {want, 1}) {
+        for (int per_cu : {3, want, 1}) {
             for (int id = 0; id < algo_count(); ++id) {
                 const Algo& a = algo_at(id);
                 if (a.kind == 2 && a.tile_t == 16 && a.param == per_cu && algo_feasible(id, N, T, K, lim)) return id;
@@ -716,6 +719,18 @@ int w4a16_probe_read(w4a16_handle* h, const void* src, size_t bytes, void* strea
     if (int rc = check_device(h)) return rc;
     const hipError_t e = launch_probe_read(src, bytes, h->sync + 64 * 40, h->cus, (hipStream_t)stream);
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "probe_read");
+}
+
+int w4a16_probe_stream(w4a16_handle* h, const void* src, size_t bytes, int wg_per_cu, int in_flight, int hint, void* stream)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    if (!src || !aligned16(src)) return fail(W4A16_EARG, "probe_stream: src must be a 16-byte aligned device pointer");
+    if (!probe_stream_config_ok(wg_per_cu, in_flight, hint))
+        return fail(W4A16_EARG, "probe_stream: wg_per_cu is 1, 2 or 4, in_flight 2, 4, 8 or 16, hint 0, 1 or 2");
+    if (h->cus > 256) return fail(W4A16_ESHAPE, "probe_stream: more than 256 CUs");
+    if (int rc = check_device(h)) return rc;
+    const hipError_t e = launch_probe_stream(src, bytes, h->sync + 64 * 40, h->cus, wg_per_cu, in_flight, hint, (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "probe_stream");
 }
 
 int w4a16_probe_barrier(w4a16_handle* h, int iters, int tree, void* stream)

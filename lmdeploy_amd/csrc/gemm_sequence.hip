@@ -115,7 +115,7 @@ __global__ void __launch_bounds__(64 * kWaves) sequence_kernel(const SeqArgs a)
             // this wave's output stores of the previous unit are complete (written through to memory)
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             const Strip st = strip_of(NT, strips, passes, pass, bx);
-            StripParams p{g.C, g.A, g.X, g.Q, g.R, g.N, a.T, g.K, 0, 0, g.epilogue};
+            StripParams p{g.C, g.A, g.X, g.Q, g.R, g.N, a.T, g.K, 0, 0, g.epilogue, 1};
             // called by every wave once its first weight loads are on their way
             auto ready = [&]() {
                 workgroup_barrier();  // every wave has drained its stores and is done with the sums in LDS

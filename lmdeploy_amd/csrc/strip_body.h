@@ -36,6 +36,7 @@ struct StripParams {
     int             base;  // column tiles of a narrow strip
     int             rem;   // the first `rem` strips have base + 1
     int             epilogue;  // read by kernels whose epilogue is chosen at run time (EPI == kEpiRuntime)
+    int             passes;    // strips per workgroup, one after the other (strip number = pass * workgroups + workgroup)
 };
 
 constexpr int kEpiRuntime = 3;  // template value: take the epilogue from StripParams

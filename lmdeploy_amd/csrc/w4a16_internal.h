@@ -116,6 +116,11 @@ hipError_t launch_from_reference(uint32_t* dst, const uint32_t* ref, int m, int 
 
 // measurement aid (probe.hip): a plain streaming read of `bytes`; sink = at least 8 * cus words
 hipError_t launch_probe_read(const void* src, size_t bytes, void* sink, int cus, hipStream_t st);
+// the same with the GEMM kernels' load pipeline: `in_flight` (2, 4, 8, 16) loads of 16 bytes per lane kept in
+// flight by count, `wg_per_cu` (1, 2, 4) workgroups of eight waves per CU, hint 0 none / 1 nt / 2 sc0 sc1
+bool       probe_stream_config_ok(int wg_per_cu, int in_flight, int hint);
+hipError_t launch_probe_stream(const void* src, size_t bytes, void* sink, int cus, int wg_per_cu, int in_flight, int hint,
+                               hipStream_t st);
 
 // decode (skinny) kernels
 bool       decode_feasible(const DecodeConfig& cf, int N, int T, int K);

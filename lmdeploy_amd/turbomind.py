@@ -204,6 +204,12 @@ class GemmS4F16:
         """Measurement aid: a plain streaming read of tensor `t`, launched like the decode kernels."""
         check(lib.w4a16_probe_read(self._h, _ptr(t), t.numel() * t.element_size(), _stream() if stream is None else stream))
 
+    def probe_stream(self, t, wg_per_cu: int, in_flight: int, hint: int, stream: Optional[int] = None) -> None:
+        """Measurement aid: the same read with the GEMM kernels' load pipeline (`in_flight` 16-byte loads per
+        lane waited for by count, `wg_per_cu` workgroups per CU, hint 0 plain / 1 non-temporal / 2 system scope)."""
+        check(lib.w4a16_probe_stream(self._h, _ptr(t), t.numel() * t.element_size(), wg_per_cu, in_flight, hint,
+                                     _stream() if stream is None else stream))
+
     def probe_barrier(self, iters: int, tree: bool = True, stream: Optional[int] = None) -> None:
         """Measurement aid: one persistent launch that crosses `iters` device-wide barriers and nothing else."""
         check(lib.w4a16_probe_barrier(self._h, iters, int(tree), _stream() if stream is None else stream))

@@ -255,14 +255,16 @@ def algo_table(tm, gemm):
     return {m.id: (m.kind, m.tile_t, m.slices) for m in ms}
 
 
-@pytest.mark.parametrize("N", [16384, 32768, 22016, 17600, 12288])
+@pytest.mark.parametrize("N", [16384, 32768, 22016, 17600, 12288, 36864, 57344])
 def test_strip_kernels_on_wide_matrices(tm, gemm, algo_table, N):
     """Strips of several column tiles (2 to 8 per workgroup, even and uneven deals of the column tiles to
-    256 and 512 workgroups), every strip configuration forced by id, few groups (so that some waves of a
-    workgroup have none), 16- and 32-token variants, every epilogue."""
+    256 and 512 workgroups, and - for more than 2048 column tiles - to 256 workgroups that take two strips one
+    after the other), every strip configuration forced by id, few groups (so that some waves of a workgroup have
+    none), 16- and 32-token variants, every epilogue."""
     K = 256
     strips = [i for i, (kind, _, _) in algo_table.items() if kind == 2]
-    assert len(strips) == 4
+    assert len(strips) == 5
+    in_turn = sorted(i for i in strips if algo_table[i][1] == 16)[2]   # one workgroup per CU, several strips in turn
     Ts = (1, 8, 16, 20, 32)
     d = O.make_inputs(4000 + N, max(Ts), K, N, residual=True)
     A, Q = convert(tm, d, N, K)
@@ -278,11 +280,12 @@ def test_strip_kernels_on_wide_matrices(tm, gemm, algo_table, N):
                     got = run(tm, gemm, dd, A, Q, T, K, N, kind, algo)
                 except tm.W4A16Error as e:
                     assert e.code == -2, e       # the 32-token strips do not take 16 tokens or fewer
-                    assert algo_table[algo][1] == 32 and T <= 16, (algo, T)
+                    # ... and the strips-in-turn kernel only takes matrices too wide for one strip of 8 tiles per CU
+                    assert (algo_table[algo][1] == 32 and T <= 16) or (algo == in_turn and N // 16 <= 2048), (algo, T)
                     continue
                 ran += 1
                 assert_close(got, want, (N, T, kind, algo))
-    assert ran >= 3 * (3 * 2 + 2 * 4)
+    assert ran >= 3 * (3 * 2 + 2 * 4) + (3 * 5 if N // 16 > 2048 else 0)
 
 
 @pytest.mark.parametrize("name,K,N,kind", [("qkv", 4096, 12288, 0), ("gate_up", 4096, 22016, 1)])

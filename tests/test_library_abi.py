@@ -141,6 +141,8 @@ def test_static_and_sequence_argument_validation(L):
     assert lib.w4a16_sequence_status(None, None) == L.EARG
     assert lib.w4a16_probe_read(None, P, 1024, None) == L.EARG
     assert lib.w4a16_probe_barrier(None, 10, 1, None) == L.EARG
+    assert lib.w4a16_probe_stream(None, P, 1024, 1, 4, 1, None) == L.EARG
+    assert lib.w4a16_probe_stream(FAKE, P, 1024, 3, 4, 1, None) == L.EARG and "wg_per_cu" in err(L)
 
 
 def test_deploy_entry_point_validation(L):
