@@ -32,6 +32,7 @@ extern "C" {
 #define W4A16_EALGO (-5)     /* algo_id out of range                         */
 #define W4A16_ESCRATCH (-6)  /* the split-K scratch this launch needs is not available */
 #define W4A16_ETIMEOUT (-7)  /* a device-wide barrier of w4a16_gemm_sequence gave up       */
+#define W4A16_ETUNING (-8)   /* a tuning file was written by another library version or GPU */
 
 /* epilogues; 0 and 1 are GemmS4F16::Type (gemm_s4_f16.h:23-27), 2 is an extension */
 #define W4A16_GEMM 0
@@ -104,8 +105,8 @@ int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const voi
  * tiles) fails with W4A16_ESCRATCH.  It calls no allocating routine; the buffer's device address
  * is looked up (hipGetSymbolAddress) by the first call on a device or by w4a16_create.  All calls
  * on one GPU share the one buffer: calls that can overlap on the GPU (different streams, or
- * different threads) race, so order them on one stream.  The counters are cleared by a small fill
- * kernel before every launch that uses them. */
+ * different threads) race, so order them on one stream.  The counters a launch will use are cleared by
+ * a small fill kernel before it. */
 int w4a16_gemm_static(void* C, const void* A, const void* X, const void* Q, const void* R, int n_out, int tokens,
                       int k, int group_size, int epilogue, int algo_id, void* stream);
 
@@ -188,6 +189,16 @@ int w4a16_pick(const w4a16_handle* h, int n_out, int tokens, int k);
 
 /* Forgets every measurement remembered by `w4a16_measure` on this handle. */
 int w4a16_clear_tuning(w4a16_handle* h);
+
+/* Writes what w4a16_measure has remembered on this handle to a text file, and reads such a file back into a
+ * handle, so that a machine measures its shapes once (boxes of one GPU model have differed by up to 19 % on the
+ * same kernel, and with them the best choice).  The file names the library version, the CU count of the device
+ * and the size of the kernel table; w4a16_load_tuning refuses a file whose three do not match the running
+ * library and the handle's device (W4A16_ETUNING, nothing loaded).  Both return the number of shapes written /
+ * taken over (entries whose kernel cannot run the shape are skipped), or a negative error.  An extension like
+ * w4a16_pick: the reference's Measure only reports (gemm_s4_f16.cu:98-169).  Host-only. */
+int w4a16_save_tuning(const w4a16_handle* h, const char* path);
+int w4a16_load_tuning(w4a16_handle* h, const char* path);
 
 /* Number of kernels `w4a16_gemm` can dispatch to (valid algo_id are 0 .. count-1). */
 int w4a16_algo_count(void);

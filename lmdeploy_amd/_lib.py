@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # W4A16_LIB overrides the in-tree library (e.g. to try a differently tuned build)
 LIB_PATH = os.environ.get("W4A16_LIB") or os.path.join(_HERE, "lib", "libw4a16.so")
 
-OK, EGROUP, ESHAPE, EHIP, EARG, EALGO, ESCRATCH, ETIMEOUT = 0, -1, -2, -3, -4, -5, -6, -7
+OK, EGROUP, ESHAPE, EHIP, EARG, EALGO, ESCRATCH, ETIMEOUT, ETUNING = 0, -1, -2, -3, -4, -5, -6, -7, -8
 GEMM, FUSED_SILU_FFN, FUSED_ADD = 0, 1, 2
 SEQ_PERSISTENT = 1
 
@@ -53,6 +53,8 @@ SIGNATURES = {
     "w4a16_algo_count": (c_int, []),
     "w4a16_pick": (c_int, [c_void_p, c_int, c_int, c_int]),
     "w4a16_clear_tuning": (c_int, [c_void_p]),
+    "w4a16_save_tuning": (c_int, [c_void_p, c_char_p]),
+    "w4a16_load_tuning": (c_int, [c_void_p, c_char_p]),
     "w4a16_convert_s4_k_m8": (c_int, [c_void_p] * 6 + [c_int] * 3 + [c_void_p]),
     "w4a16_deploy_qkv": (c_int, [c_void_p, c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p)] + [c_int] * 5
                          + [c_void_p]),

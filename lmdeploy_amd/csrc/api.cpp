@@ -373,20 +373,66 @@ int w4a16_clear_tuning(w4a16_handle* h)
     return W4A16_OK;
 }
 
+// File format: a header line that names the library version, the CU count of the device and the size of the kernel
+// table - a measurement is only worth anything for that combination - then one line "n_out tokens k algo_id" per shape.
+int w4a16_save_tuning(const w4a16_handle* h, const char* path)
+{
+    if (!h || !path) return fail(W4A16_EARG, "save_tuning: null argument");
+    FILE* f = fopen(path, "w");
+    if (!f) return fail(W4A16_EARG, "save_tuning: cannot open %s for writing", path);
+    fprintf(f, "w4a16-tuning 1 \"%s\" cus=%d algos=%d\n", w4a16_version(), h->cus, algo_count());
+    for (const auto& kv : h->tuned)
+        fprintf(f, "%d %d %d %d\n", std::get<0>(kv.first), std::get<1>(kv.first), std::get<2>(kv.first), kv.second);
+    const bool bad = ferror(f) != 0;
+    if (fclose(f) != 0 || bad) return fail(W4A16_EARG, "save_tuning: writing %s failed", path);
+    return (int)h->tuned.size();
+}
+
+int w4a16_load_tuning(w4a16_handle* h, const char* path)
+{
+    if (!h || !path) return fail(W4A16_EARG, "load_tuning: null argument");
+    FILE* f = fopen(path, "r");
+    if (!f) return fail(W4A16_EARG, "load_tuning: cannot open %s", path);
+    char version[128] = "";
+    int  cus = 0, algos = 0, fmt = 0;
+    const int got = fscanf(f, "w4a16-tuning %d \"%127[^\"]\" cus=%d algos=%d", &fmt, version, &cus, &algos);
+    if (got != 4 || fmt != 1) {
+        fclose(f);
+        return fail(W4A16_EARG, "load_tuning: %s is not a tuning file", path);
+    }
+    if (strcmp(version, w4a16_version()) != 0 || cus != h->cus || algos != algo_count()) {
+        fclose(f);
+        return fail(W4A16_ETUNING, "load_tuning: %s was measured with \"%s\" on %d CUs (%d kernels); this is \"%s\" on %d CUs "
+                                   "(%d kernels): ignored", path, version, cus, algos, w4a16_version(), h->cus, algo_count());
+    }
+    int n_out, tokens, k, id, loaded = 0;
+    while (fscanf(f, "%d %d %d %d", &n_out, &tokens, &k, &id) == 4) {
+        if (n_out <= 0 || tokens <= 0 || k <= 0 || id < 0 || id >= algo_count()) continue;
+        if (!algo_feasible(id, n_out, tokens, k, h->scratch)) continue;
+        h->tuned[std::make_tuple(n_out, tokens, k)] = id;
+        ++loaded;
+    }
+    fclose(f);
+    return loaded;
+}
+
 int w4a16_algo_count(void)
 {
     return algo_count();
 }
 
-int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R, int n_out,
-               int tokens, int k, int group_size, int epilogue, int algo_id, void* stream)
+// What w4a16_gemm decides before it launches: the kernel and the scratch it may use.  Everything that can
+// fail for reasons other than the launch itself happens here, so that a list of GEMMs can be planned as a
+// whole before the first of them is enqueued.
+struct GemmPlan {
+    int     algo;
+    Scratch sc;
+};
+
+int plan_gemm(w4a16_handle* h, const void* C, const void* R, int n_out, int tokens, int k, int epilogue, int algo_id,
+              hipStream_t st, GemmPlan* out)
 {
-    if (!h) return fail(W4A16_EARG, "null handle");
-    const int chk = check_gemm_args(C, A, X, Q, R, n_out, tokens, k, group_size, epilogue);
-    if (chk < 0) return chk;
-    if (chk > 0) return W4A16_OK;
     if (algo_id >= algo_count()) return fail(W4A16_EALGO, "algo_id %d out of range (0..%d)", algo_id, algo_count() - 1);
-    if (int rc = check_device(h)) return rc;
     const bool chosen = algo_id >= 0;
     if (!chosen) algo_id = pick_for(h, n_out, tokens, k);
     if (algo_id < 0 || !algo_feasible(algo_id, n_out, tokens, k, h->scratch))
@@ -394,7 +440,7 @@ int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const voi
     Scratch sc = h->scratch;
     if (algo_scratch_bytes(algo_id, n_out, tokens, k, sc) > 0) {
         bool have = false;
-        if (int rc = ensure_workspace(h, (hipStream_t)stream, &have)) return rc;
+        if (int rc = ensure_workspace(h, st, &have)) return rc;
         sc = h->scratch;
         if (!have) {
             // the stream is being captured and this handle has never split K before: nothing can be allocated now
@@ -406,9 +452,25 @@ int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const voi
         }
     }
     if (int rc = check_prefill_alignment(algo_id, C, R, epilogue)) return rc;
+    out->algo = algo_id;
+    out->sc   = sc;
+    return W4A16_OK;
+}
+
+int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const void* Q, const void* R, int n_out,
+               int tokens, int k, int group_size, int epilogue, int algo_id, void* stream)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    const int chk = check_gemm_args(C, A, X, Q, R, n_out, tokens, k, group_size, epilogue);
+    if (chk < 0) return chk;
+    if (chk > 0) return W4A16_OK;
+    if (algo_id >= algo_count()) return fail(W4A16_EALGO, "algo_id %d out of range (0..%d)", algo_id, algo_count() - 1);
+    if (int rc = check_device(h)) return rc;
+    GemmPlan plan{};
+    if (int rc = plan_gemm(h, C, R, n_out, tokens, k, epilogue, algo_id, (hipStream_t)stream, &plan)) return rc;
     GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
                n_out,        tokens,             k,                  epilogue};
-    const hipError_t e = algo_launch(algo_id, g, sc, (hipStream_t)stream);
+    const hipError_t e = algo_launch(plan.algo, g, plan.sc, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "w4a16_gemm launch");
     return W4A16_OK;
 }
@@ -437,7 +499,9 @@ int w4a16_gemm_static(void* C, const void* A, const void* X, const void* Q, cons
     const hipStream_t st = (hipStream_t)stream;
     if (algo_scratch_bytes(algo_id, n_out, tokens, k, sc) > 0) {
         // every call on this GPU shares the array, whatever an earlier (perhaps aborted) call left in it
-        if (const hipError_t e = clear_counters(sc, st); e != hipSuccess) return hip_fail(e, "w4a16_gemm_static clear");
+        // (only the counters this launch will use: one per output tile or column block, never more than workgroups)
+        const int used = std::min(sc.cnt_len, algo_grid(algo_id, n_out, tokens, k, sc));
+        if (const hipError_t e = clear_counters(sc, used, st); e != hipSuccess) return hip_fail(e, "w4a16_gemm_static clear");
     }
     GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
                n_out,        tokens,             k,                  epilogue};
@@ -462,11 +526,19 @@ int w4a16_gemm_sequence(w4a16_handle* h, const w4a16_gemm_desc* gemms, int count
     if (tokens == 0 || count == 0) return W4A16_OK;
     if (int rc = check_device(h)) return rc;
     if (!(flags & W4A16_SEQ_PERSISTENT) || tokens > 16 || count == 1) {
-        // one launch per GEMM; stream order gives the dependencies
+        // One launch per GEMM; stream order gives the dependencies.  Every GEMM is planned (kernel, workspace,
+        // alignment) before the first one is launched: a list that cannot run as a whole runs not at all.
+        std::vector<GemmPlan> plans(count);
         for (int i = 0; i < count; ++i) {
             const w4a16_gemm_desc& d = gemms[i];
-            const int rc = w4a16_gemm(h, d.C, d.A, d.X, d.Q, d.R, d.n_out, tokens, d.k, group_size, d.epilogue, -1, stream);
-            if (rc != W4A16_OK) return rc;
+            if (int rc = plan_gemm(h, d.C, d.R, d.n_out, tokens, d.k, d.epilogue, -1, (hipStream_t)stream, &plans[i])) return rc;
+        }
+        for (int i = 0; i < count; ++i) {
+            const w4a16_gemm_desc& d = gemms[i];
+            GemmArgs g{(uint16_t*)d.C, (const uint32_t*)d.A, (const uint16_t*)d.X, (const uint32_t*)d.Q, (const uint16_t*)d.R,
+                       d.n_out,        tokens,                d.k,                  d.epilogue};
+            const hipError_t e = algo_launch(plans[i].algo, g, plans[i].sc, (hipStream_t)stream);
+            if (e != hipSuccess) return hip_fail(e, "w4a16_gemm_sequence launch");  // (the launch itself: earlier GEMMs are enqueued)
         }
         return W4A16_OK;
     }
@@ -749,7 +821,7 @@ const char* w4a16_last_error(void)
 
 const char* w4a16_version(void)
 {
-    return "w4a16-gfx950 0.2";
+    return "w4a16-gfx950 0.3";
 }
 
 }  // extern "C"

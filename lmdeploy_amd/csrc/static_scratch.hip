@@ -8,6 +8,7 @@
 // device with that device current, and only that address is ever handed to a kernel.
 #include "w4a16_internal.h"
 
+#include <algorithm>
 #include <mutex>
 
 namespace w4a16 {
@@ -57,11 +58,12 @@ hipError_t static_scratch(Scratch* out)
     return hipSuccess;
 }
 
-hipError_t clear_counters(const Scratch& sc, hipStream_t st)
+hipError_t clear_counters(const Scratch& sc, int n, hipStream_t st)
 {
-    if (!sc.cnt || sc.cnt_len <= 0) return hipSuccess;
+    n = std::min(n, sc.cnt_len);
+    if (!sc.cnt || n <= 0) return hipSuccess;
     // a kernel, not hipMemsetAsync: the call may be recorded into a graph
-    return launch_kernel(fill_zero_kernel, dim3((sc.cnt_len + 255) / 256), dim3(256), 0, st, sc.cnt, sc.cnt_len);
+    return launch_kernel(fill_zero_kernel, dim3((n + 255) / 256), dim3(256), 0, st, sc.cnt, n);
 }
 
 }  // namespace w4a16

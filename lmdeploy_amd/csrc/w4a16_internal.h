@@ -96,8 +96,8 @@ hipError_t algo_launch(int id, const GemmArgs& a, const Scratch& sc, hipStream_t
 constexpr size_t kStaticCounters       = 4096;
 constexpr size_t kStaticWorkspaceBytes = 8u << 20;
 hipError_t static_scratch(Scratch* out);
-// zeroes the arrival counters of `sc` with a fill kernel on `st`
-hipError_t clear_counters(const Scratch& sc, hipStream_t st);
+// zeroes the first `n` arrival counters of `sc` with a fill kernel on `st`
+hipError_t clear_counters(const Scratch& sc, int n, hipStream_t st);
 
 hipError_t launch_convert(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* A_src, const uint16_t* scales,
                           const uint32_t* qzeros, int m, int k, hipStream_t st);

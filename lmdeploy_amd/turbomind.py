@@ -11,6 +11,7 @@ All work is queued on torch's current stream.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import List, Optional
 
 import torch
@@ -221,3 +222,11 @@ class GemmS4F16:
 
     def clear_tuning(self) -> None:
         check(lib.w4a16_clear_tuning(self._h))
+
+    def save_tuning(self, path: str) -> int:
+        """Writes the kernels `Measure` found fastest to a text file; returns the number of shapes."""
+        return check(lib.w4a16_save_tuning(self._h, os.fsencode(path)))
+
+    def load_tuning(self, path: str) -> int:
+        """Reads such a file (W4A16Error code -8 if it was written by another library version or GPU)."""
+        return check(lib.w4a16_load_tuning(self._h, os.fsencode(path)))

@@ -359,6 +359,23 @@ def test_llama7b_prefill_shapes_sampled_rows(tm, gemm, name, K, N, kind):
     assert_close(got[rows], want, name)
 
 
+def test_llama7b_o_prefill_every_output_row(tm, gemm):
+    # The sampled comparisons of the T = 2048 shapes rest on this one: the smallest of them (o, 4096 x 4096)
+    # with all 2048 x 4096 outputs held against the oracle, for the default kernel and every large prefill tile.
+    T, K, N = 2048, 4096, 4096
+    d = O.make_inputs(SEED["o"] + 2, T, K, N)
+    A, Q = convert(tm, d, N, K)
+    W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], 128)
+    want = O.epilogue(O.gemm_acc(d["X"], W), 0)
+    assert_close(run(tm, gemm, d, A, Q, T, K, N, 0), want, "o, default kernel")
+    ms = gemm.Measure(torch.empty(T, N, dtype=torch.float16, device="cuda"), A, dev(d["X"]), Q, N, T, K, 128)
+    gemm.clear_tuning()
+    large = [m.id for m in ms if m.feasible and m.kind == 1 and m.slices == 1 and m.tile_t >= 128]
+    assert len(large) >= 3
+    for algo in large:
+        assert_close(run(tm, gemm, d, A, Q, T, K, N, 0, algo), want, ("o", algo))
+
+
 LLAMA70B = [("qkv70", 8192, 10240, 0), ("o70", 8192, 8192, 0), ("gate_up70", 8192, 57344, 1), ("down70", 28672, 8192, 2)]
 
 
@@ -640,3 +657,39 @@ def test_measure_reports_all_kernels(tm, gemm):
     assert gemm.pick(N, T, K) == heuristic
     with pytest.raises(tm.W4A16Error):
         gemm.pick(N + 8, T, K)
+
+
+def test_measured_choices_survive_in_a_file(tm, tmp_path):
+    """w4a16_measure -> w4a16_save_tuning -> a fresh handle -> w4a16_load_tuning: the fresh handle then picks
+    what was measured; a file written for another library version or CU count is refused and changes nothing."""
+    T, K, N = 24, 1024, 512
+    d = O.make_inputs(8800, T, K, N)
+    A, Q = convert(tm, d, N, K)
+    g1 = tm.GemmS4F16()
+    ms = g1.Measure(torch.empty(T, N, dtype=torch.float16, device="cuda"), A, dev(d["X"]), Q, N, T, K, 128)
+    fastest = ms[0].id
+    assert g1.pick(N, T, K) == fastest
+    path = str(tmp_path / "tuning.txt")
+    assert g1.save_tuning(path) == 1
+    g2 = tm.GemmS4F16()
+    heuristic = g2.pick(N, T, K)
+    assert g2.load_tuning(path) == 1
+    assert g2.pick(N, T, K) == fastest
+    want = O.gemm_s4_f16(d["X"], d["qweight"], d["qzeros"], d["scales"], 128)
+    assert_close(run(tm, g2, d, A, Q, T, K, N), want, "tuned pick")
+    # another version / another GPU: refused
+    text = open(path).read()
+    other = str(tmp_path / "other.txt")
+    open(other, "w").write(text.replace("cus=", "cus=9", 1))
+    g3 = tm.GemmS4F16()
+    with pytest.raises(tm.W4A16Error) as e:
+        g3.load_tuning(other)
+    assert e.value.code == -8 and g3.pick(N, T, K) == heuristic
+    open(other, "w").write("hello\n")
+    with pytest.raises(tm.W4A16Error) as e:
+        g3.load_tuning(other)
+    assert e.value.code == -4
+    # an entry whose kernel cannot run its shape is skipped, the others are taken
+    lines = text.splitlines()
+    open(other, "w").write("\n".join([lines[0], "72 4 256 0", lines[1]]) + "\n")
+    assert g3.load_tuning(other) == 1 and g3.pick(N, T, K) == fastest

@@ -139,6 +139,9 @@ def test_static_and_sequence_argument_validation(L):
     assert seq(FAKE, one, 2, 0, 128, L.SEQ_PERSISTENT, None) == L.OK   # no tokens
     assert lib.w4a16_set_barrier_timeout(None, 1.0) == L.EARG
     assert lib.w4a16_sequence_status(None, None) == L.EARG
+    assert lib.w4a16_save_tuning(None, b"/tmp/x") == L.EARG and lib.w4a16_load_tuning(None, b"/tmp/x") == L.EARG
+    assert lib.w4a16_save_tuning(FAKE, None) == L.EARG and lib.w4a16_load_tuning(FAKE, None) == L.EARG
+    assert lib.w4a16_load_tuning(FAKE, b"/nonexistent/dir/tuning.txt") == L.EARG and "cannot open" in err(L)
     assert lib.w4a16_probe_read(None, P, 1024, None) == L.EARG
     assert lib.w4a16_probe_barrier(None, 10, 1, None) == L.EARG
     assert lib.w4a16_probe_stream(None, P, 1024, 1, 4, 1, None) == L.EARG

@@ -166,3 +166,26 @@ def test_a_barrier_that_gives_up_is_reported_and_every_workgroup_still_finishes(
         close(C.cpu().numpy(), want, "after the timeout")
     with pytest.raises(tm.W4A16Error):
         gemm.set_barrier_timeout(-1.0)
+
+
+def test_a_list_that_cannot_run_as_a_whole_launches_nothing(tm):
+    """Every GEMM of a list is planned (kernel, workspace, alignment) before the first one is launched: a second
+    GEMM whose output pointer is misaligned for the MFMA kernels (8 bytes above 32 tokens) fails the call, and the
+    first GEMM's output is still untouched."""
+    T, K, N = 512, 1024, 2048
+    d = O.make_inputs(9100, T, K, N)
+    A, Q = convert(tm, d, N, K)
+    X = dev(d["X"])
+    C0 = torch.full((T, N), float("nan"), dtype=torch.float16, device="cuda")
+    buf = torch.zeros(T * N + 8, dtype=torch.float16, device="cuda")
+    C1 = buf[2:2 + T * N].view(T, N)          # 4-byte aligned only
+    gemm = tm.GemmS4F16()
+    with pytest.raises(tm.W4A16Error, match="misaligned") as e:
+        gemm.sequence([(C0, A, X, Q, N, K, 0, None, False), (C1, A, X, Q, N, K, 0, None, False)], T)
+    assert e.value.code == -4
+    torch.cuda.synchronize()
+    assert torch.isnan(C0).all()
+    gemm.sequence([(C0, A, X, Q, N, K, 0, None, False)], T)
+    torch.cuda.synchronize()
+    want = O.gemm_s4_f16(d["X"], d["qweight"], d["qzeros"], d["scales"], 128)
+    assert O.max_abs_rel(C0.cpu().numpy(), want) <= 1e-2

@@ -66,6 +66,48 @@ def test_static_scratch_entry_point_equals_the_handle_entry_point():
     assert used_scratch >= 24
 
 
+def test_static_scratch_decode_kernels_that_split_k_across_workgroups():
+    """Narrow matrices at up to 16 tokens take the column-block decode kernel with K split across workgroups,
+    whose partial tiles and counters also come from the static buffer: every such configuration, and the default
+    choice, bit for bit against the handle's workspace; then replayed from a graph."""
+    import lmdeploy_amd.turbomind as tm
+    gemm = tm.GemmS4F16()
+    K, N, T = 5632, 1024, 12
+    d = O.make_inputs(5180, T, K, N, residual=True)
+    A, Q = convert(tm, d, N, K)
+    X, R = dev(d["X"]), dev(d["R"])
+    ms = gemm.Measure(torch.empty((T, N), dtype=torch.float16, device="cuda"), A, X, Q, N, T, K, 128, gemm.kGemm)
+    gemm.clear_tuning()
+    # a column-block kernel that launches more workgroups than it has column blocks splits K across them
+    split = [m.id for m in ms if m.feasible and m.kind == 0 and m.grid > N // m.tile_n]
+    assert len(split) >= 3, split
+    picked = gemm.pick(N, T, K)
+    assert picked in split, (picked, split)      # what algo_id = -1 runs for this shape
+    want = O.gemm_s4_f16(d["X"], d["qweight"], d["qzeros"], d["scales"], 128, O.EPI_ADD, d["R"])
+    outs = []
+    for algo in [-1] + split:
+        Ch = torch.full((T, N), float("nan"), dtype=torch.float16, device="cuda")
+        Cs = torch.full((T, N), float("nan"), dtype=torch.float16, device="cuda")
+        gemm.Run(Ch, A, X, Q, N, T, K, 128, gemm.kFusedAdd, algo, residual=R)
+        tm.gemm_static(Cs, A, X, Q, N, T, K, 128, gemm.kFusedAdd, algo, residual=R)
+        torch.cuda.synchronize()
+        assert O.max_abs_rel(Cs.cpu().numpy(), want) <= TOL, algo
+        assert torch.equal(Cs.view(torch.int16), Ch.view(torch.int16)), algo
+        outs.append(Cs)
+    stream = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    caps = [torch.empty((T, N), dtype=torch.float16, device="cuda") for _ in outs]
+    with torch.cuda.graph(g, stream=stream):
+        st = torch.cuda.current_stream().cuda_stream
+        for algo, C in zip([-1] + split, caps):
+            tm.gemm_static(C, A, X, Q, N, T, K, 128, gemm.kFusedAdd, algo, residual=R, stream=st)
+    for rep in range(3):
+        g.replay()
+        torch.cuda.synchronize()
+        for C, E in zip(caps, outs):
+            assert torch.equal(C.view(torch.int16), E.view(torch.int16)), rep
+
+
 def test_static_scratch_rejects_what_does_not_fit():
     import lmdeploy_amd.turbomind as tm
     gemm = tm.GemmS4F16()
