@@ -106,6 +106,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=96)
     ap.add_argument("--warmup", type=int, default=24)
+    ap.add_argument("--repeats", type=int, default=9,
+                    help="the timed region of --steps steps is measured this many times in a row; the median is reported")
     ap.add_argument("--copies", type=int, default=12,
                     help="distinct sets of 16 weight matrices (one per GEMM of a step) the steps rotate through")
     ap.add_argument("--cold-gib", type=float, default=1.25,
@@ -119,10 +121,11 @@ def main():
     ap.add_argument("--no-sustained", action="store_true", help="skip the power / clock reading under a sustained prefill load")
     ap.add_argument("--sustained-seconds", type=float, default=4.0)
     ap.add_argument("--seconds", type=float, default=8.0, help="duration of the sustain-* probes")
-    ap.add_argument("--probe", choices=["decode", "prefill", "decode-o", "sustain-prefill",
+    ap.add_argument("--probe", choices=["decode", "prefill", "decode-o", "decode-70b", "sustain-prefill",
                                         "sustain-decode", "sustain-dense"],
                     help="decode / prefill / decode-o: run only the named kernel (gate_up decode / gate_up at T=2048 / o "
                          "decode) plus a plain 256 MiB elementwise kernel, eagerly, for `rocprofv3 --pmc` (no JSON line).  "
+                         "decode-70b: the same for the Llama-2-70B gate_up and down decode kernels at T=1 and T=16.  "
                          "sustain-prefill / sustain-decode / sustain-dense: "
                          "keep launching gate_up (T=2048 / T=8 / torch.matmul fp16 at T=2048) for --seconds and print the "
                          "rate once a second, so that the engine clock under that load can be read beside it "
@@ -149,7 +152,9 @@ def main():
     for name, K, N, epi in LAYER_7B:
         per_copy = K * N // 2 + (K // GROUP) * N * 4
         n = max(len(DECODE_T) * n_sets, N_LAYERS, int(args.cold_gib * 2 ** 30 / per_copy) + 1)
-        if args.probe:
+        if args.probe == "decode-70b":
+            n = 1
+        elif args.probe:
             n = max(8, int(args.cold_gib * 2 ** 30 / per_copy) + 1) if name in ("gate_up", "o") else 1
         weights[name] = [make_weights(tm, torch, gen, name, K, N) for _ in range(n)]
     Tmax = max(max(DECODE_T), PREFILL_T)
@@ -180,18 +185,30 @@ def main():
             runners.append(lambda g=g, keep=keep: g.replay())
         return runners
 
-    def timed(runner, steps, warmup):
+    def timed_all(runner, steps, warmup, repeats):
+        """`warmup` untimed calls, then `repeats` timed regions of exactly `steps` calls each (HIP events on the
+        stream the graphs replay on, a synchronisation on both sides of every region); ms per region."""
+        out, n = [], 0
         with torch.cuda.stream(stream):
-            for i in range(warmup):
-                runner[i % len(runner)]()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            torch.cuda.synchronize()
-            e0.record(stream)
-            for i in range(steps):
-                runner[(warmup + i) % len(runner)]()
-            e1.record(stream)
-            torch.cuda.synchronize()
-        return e0.elapsed_time(e1)   # ms
+            for _ in range(warmup):
+                runner[n % len(runner)]()
+                n += 1
+            for _ in range(repeats):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                torch.cuda.synchronize()
+                e0.record(stream)
+                for _ in range(steps):
+                    runner[n % len(runner)]()
+                    n += 1
+                e1.record(stream)
+                torch.cuda.synchronize()
+                out.append(e0.elapsed_time(e1))
+        return out
+
+    def timed(runner, steps, warmup, repeats=1):
+        """Median over `repeats` timed regions of `steps` calls, in ms per region."""
+        ms = sorted(timed_all(runner, steps, warmup, repeats))
+        return ms[len(ms) // 2]
 
     if args.probe and args.probe.startswith("sustain-"):
         K, N, _ = shape["gate_up"]
@@ -220,6 +237,34 @@ def main():
                 algorithmic_bytes(T, K, N, 0 if dense_w is not None else 1) / us / 1e3), flush=True)
         return
 
+    if args.probe == "decode-70b":
+        # calibration kernel, then gate_up (strips of 7 tiles, SiLU) and down (strips of 2, residual) of Llama-2-70B,
+        # every weight copy once at T = 1 and once at T = 16, cold
+        src = torch.zeros(64 * 2 ** 20, dtype=torch.int32, device="cuda")   # 256 MiB
+        dst = torch.empty_like(src)
+        X70 = {K: torch.randn((16, K), device="cuda", generator=gen).half() for K in (8192, 28672)}
+        Res70 = torch.randn((16, 8192), device="cuda", generator=gen).half()
+        with torch.cuda.stream(stream):
+            for _ in range(4):
+                torch.add(src, 1, out=dst)
+        done = []
+        for name, K, N, epi in LAYER_70B:
+            if name not in ("gate_up", "down"):
+                continue
+            n = max(3, int(args.cold_gib * 2 ** 30 / (K * N // 2 + (K // GROUP) * N * 4)) + 1)
+            ws = [make_weights(tm, torch, gen, name, K, N) for _ in range(n)]
+            C = torch.empty((16, N // 2 if epi == 1 else N), dtype=torch.float16, device="cuda")
+            with torch.cuda.stream(stream):
+                for T in (1, 16):
+                    for A, Q in ws:
+                        gemm.Run(C, A, X70[K], Q, N, T, K, GROUP, epi, -1, residual=Res70 if epi == 2 else None,
+                                 stream=stream.cuda_stream)
+            torch.cuda.synchronize()
+            done.append("%d %s launches at T=1 and as many at T=16" % (n, name))
+            del ws
+        print("probe done: 4 add kernels over 268435456 bytes, " + ", ".join(done))
+        return
+
     if args.probe:
         # a plain elementwise kernel of known size calibrates FETCH_SIZE / WRITE_SIZE, then the kernel on cold weights
         src = torch.zeros(64 * 2 ** 20, dtype=torch.int32, device="cuda")   # 256 MiB
@@ -240,24 +285,31 @@ def main():
     step_bytes = sum(algorithmic_bytes(T, K, N, epi) for T in DECODE_T for _, K, N, epi in LAYER_7B)
     runner = make_runner([[(name, len(DECODE_T) * c + ti, T) for ti, T in enumerate(DECODE_T) for name, _, _, _ in LAYER_7B]
                           for c in range(n_sets)])
-    ms = timed(runner, args.steps, args.warmup)
+    # One timed region of `steps` steps lasts a few milliseconds and cannot resolve a 3 % change; the region is
+    # therefore timed `--repeats` times in a row and the median region is the one reported.
+    regions = sorted(timed_all(runner, args.steps, args.warmup, args.repeats))
+    ms = regions[len(regions) // 2]
     ms_per_step = ms / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    timing = {"regions": args.repeats, "steps_per_region": args.steps, "reported": "median region",
+              "min_ms_per_step": round(regions[0] / args.steps, 5), "max_ms_per_step": round(regions[-1] / args.steps, 5)}
 
-    def per_launch_us(name, tokens, passes=3):
-        """Average time of one launch of `name`, rotating through all of its copies (cold weights)."""
+    def per_launch_us(name, tokens, passes=3, repeats=3):
+        """Average time of one launch of `name`, rotating through all of its copies (cold weights); median of
+        `repeats` regions of `passes` rounds."""
         n = len(weights[name])
         r = make_runner([[(name, c, tokens[c % len(tokens)]) for c in range(n)]])
-        return timed(r, passes, 1) * 1e3 / (passes * n)
+        return timed(r, passes, 1, repeats) * 1e3 / (passes * n)
 
     def decode_roofline(name, traffic, what):
         K, N, epi = shape[name]
         by = sum(algorithmic_bytes(T, K, N, epi) for T in DECODE_T) / len(DECODE_T)
-        us = per_launch_us(name, DECODE_T, passes=6)
+        us = per_launch_us(name, DECODE_T, passes=4, repeats=7)
         ach = by / (us * 1e-6) / 1e9
         return {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": what,
-                "bytes_per_launch": int(by), "us_per_launch": round(us, 3)}
+                "bytes_per_launch": int(by), "us_per_launch": round(us, 3),
+                "us_per_launch_is": "median of 7 regions of 4 rounds over all weight copies"}
 
     # ---- rooflines: the dominant decode kernel (gate_up) and the one furthest below its roofline (o) ----
     roofline = decode_roofline("gate_up", TRAFFIC_DECODE_GATE_UP,
@@ -291,7 +343,7 @@ def main():
             # four launches on four weight copies per graph: the gap between graph launches
             # (several microseconds) would otherwise count as kernel time
             r = make_runner([[(name, 4 * g + c, PREFILL_T) for c in range(4)] for g in range(2)])
-            t_ms = timed(r, args.prefill_steps, 3) / args.prefill_steps / 4
+            t_ms = timed(r, args.prefill_steps, 3, 5) / args.prefill_steps / 4
             fl = flops(PREFILL_T, K, N)
             rows.append({"shape": name, "ms": round(t_ms, 4), "TFLOPs": round(fl / t_ms / 1e9, 1),
                          "frac": round(fl / t_ms / 1e9 / MFMA_PEAK_TFLOPS, 4)})
@@ -346,7 +398,7 @@ def main():
                 "frac": round(seq_bytes / ms_ / 1e6 / HBM_PEAK_GBS, 4)}
 
     seq_work = [[(name, layer, seq_T) for layer in range(N_LAYERS) for name, _, _, _ in LAYER_7B]]
-    seq_ms = timed(make_runner(seq_work), 20, 5) / 20
+    seq_ms = timed(make_runner(seq_work), 20, 5, 7) / 20
 
     def persistent(w, st):
         descs = []
@@ -356,7 +408,7 @@ def main():
             descs.append((out[name], A, X[K], Q, N, K, epi, Res if epi == 2 else None, i > 0))
         return gemm.sequence(descs, seq_T, persistent=True, stream=st)
 
-    pers_ms = timed(make_runner(seq_work, persistent), 20, 5) / 20
+    pers_ms = timed(make_runner(seq_work, persistent), 20, 5, 3) / 20
     gemm.sequence_status(stream.cuda_stream)
     layers32_m8 = dict(layers32(seq_ms, "one launch per GEMM (128 launches, one HIP graph)"), T=seq_T, layers=N_LAYERS,
                        gemms=4 * N_LAYERS,
@@ -370,15 +422,27 @@ def main():
     ceilings = None
     if not args.no_prefill:
         reads = {}
-        for mib in (8, 45, 512):
+        # (workgroups per CU, 16-byte loads in flight per lane, hint: 1 = non-temporal) of w4a16_probe_stream; the
+        # configurations that came out ahead in a full sweep (1, 2, 4 workgroups x 2, 4, 8, 16 loads x 3 hints)
+        stream_configs = [(1, 4, 1), (1, 8, 1), (2, 2, 1), (1, 4, 0), (2, 8, 1), (2, 16, 1)]
+        for mib in (8, 45, 244, 512):
             n = max(3, int(args.cold_gib * 1024 / mib) + 1)
             bufs = [torch.empty(mib << 20, dtype=torch.uint8, device="cuda") for _ in range(n)]
             for b in bufs:
                 b.zero_()
             r = make_runner([bufs], lambda w, st: [gemm.probe_read(b, stream=st) for b in w])
-            us = timed(r, 3, 1) * 1e3 / (3 * n)
-            reads["read_%dMiB" % mib] = {"us": round(us, 2), "GBps": round((mib << 20) / us / 1e3, 1),
-                                         "frac": round((mib << 20) / us / 1e3 / HBM_PEAK_GBS, 3)}
+            us = timed(r, 3, 1, 3) * 1e3 / (3 * n)
+            row = {"us": round(us, 2), "GBps": round((mib << 20) / us / 1e3, 1),
+                   "frac": round((mib << 20) / us / 1e3 / HBM_PEAK_GBS, 3)}
+            swept = {}
+            for wg, fl, hint in stream_configs:
+                r = make_runner([bufs], lambda w, st: [gemm.probe_stream(b, wg, fl, hint, stream=st) for b in w])
+                swept["wg%d_inflight%d_%s" % (wg, fl, "nt" if hint else "plain")] = round(timed(r, 3, 1, 3) * 1e3 / (3 * n), 2)
+            best = min(swept, key=swept.get)
+            row["counted_loads_us"] = swept
+            row["best"] = {"config": best, "us": swept[best], "GBps": round((mib << 20) / swept[best] / 1e3, 1),
+                           "frac": round((mib << 20) / swept[best] / 1e3 / HBM_PEAK_GBS, 3)}
+            reads["read_%dMiB" % mib] = row
             del bufs, r
         with torch.cuda.stream(stream):
             src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
@@ -419,7 +483,9 @@ def main():
         gemm.sequence_status(stream.cuda_stream)
         ceilings = dict(reads, device_wide_barrier=barrier, device_copy_512MiB_GBps=round(copy_gbs, 1),
                         dense_fp16_gemm_gate_up_T2048_TFLOPs=round(dense_tf, 1),
-                        note="read_*: w4a16_probe_read (plain streaming read, one launch per buffer in a HIP graph, cold buffers); "
+                        note="read_*: w4a16_probe_read (plain streaming read, one launch per buffer in a HIP graph, cold buffers) and, "
+                             "under counted_loads_us, w4a16_probe_stream (the GEMM kernels' load pipeline: wgN = workgroups of eight "
+                             "waves per CU, inflightN = 16-byte loads per lane kept in flight, nt = non-temporal); "
                              "device_wide_barrier: w4a16_probe_barrier, one workgroup per CU, 2000 barriers in one launch; "
                              "torch copy_ (bytes read + written); torch.matmul fp16 (hipBLASLt)")
 
@@ -442,11 +508,11 @@ def main():
                     gemm.Run(C, ws[c][0], X70[K], ws[c][1], N, T, K, GROUP, epi, -1, residual=Res70 if epi == 2 else None,
                              stream=st)
             for T in DECODE_T_70B:
-                us = timed(make_runner([[(c, T) for c in range(n)]], run70), 3, 1) * 1e3 / (3 * n)
+                us = timed(make_runner([[(c, T) for c in range(n)]], run70), 3, 1, 5) * 1e3 / (3 * n)
                 by = algorithmic_bytes(T, K, N, epi)
                 rows70.append({"shape": name, "T": T, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
                                "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 3)})
-            us = timed(make_runner([[(c, PREFILL_T) for c in range(n)]], run70), 2, 1) * 1e3 / (2 * n)
+            us = timed(make_runner([[(c, PREFILL_T) for c in range(n)]], run70), 2, 1, 3) * 1e3 / (2 * n)
             fl = flops(PREFILL_T, K, N)
             rows70.append({"shape": name, "T": PREFILL_T, "us": round(us, 1), "TFLOPs": round(fl / us / 1e6, 1),
                            "frac": round(fl / us / 1e6 / MFMA_PEAK_TFLOPS, 4)})
@@ -508,7 +574,7 @@ def main():
     line = {
         "metric": "W4A16 GEMM achieved HBM GB/s (M=1..16) + TFLOP/s (M=2048), % of roofline",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 5), "timing": timing, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "Llama-2-7B decode layer set (qkv 4096x12288, o 4096x4096, gate_up 4096x22016 +SiLU, "
                                "down 11008x4096 +residual) at T in {1,4,8,16}, group 128: 16 GEMMs per step, each on its own "

@@ -25,7 +25,7 @@ extern "C" {
 #endif
 
 #define W4A16_OK 0
-#define W4A16_EGROUP (-1)    /* unsupported group size (only 128)            */
+#define W4A16_EGROUP (-1)    /* unsupported group size (128, 64 and 32 have kernels) */
 #define W4A16_ESHAPE (-2)    /* no feasible kernel for this shape            */
 #define W4A16_EHIP (-3)      /* the HIP runtime reported an error            */
 #define W4A16_EARG (-4)      /* null pointer / negative size / bad enum      */
@@ -81,7 +81,12 @@ void w4a16_destroy(w4a16_handle* h);
  *                         (no counterpart in GemmS4F16; the add of
  *                          llama_decoder_kernels.cu:52-57 applied as in LlamaDecoder.cc:228-235)
  * algo_id < 0 selects a kernel by heuristic (gemm_s4_f16.cu:184-206 `Estimate`).
- * Requires group_size == 128, k % 128 == 0, n_out % 16 == 0, tokens >= 0; A and X aligned to 16
+ * group_size: 128 is the reference's only one (gemm_s4_f16.cu:243-245, "TODO: add more group sizes") and has
+ * the whole kernel table.  64 and 32 are an extension served by one kernel family (strips of up to four column
+ * tiles, 16 tokens per workgroup, the weights streamed once per 16 tokens): they take algo_id < 0 only
+ * (W4A16_EALGO otherwise), w4a16_measure refuses them, and a persistent w4a16_gemm_sequence runs them as one
+ * launch per GEMM.  Any other value: W4A16_EGROUP, "unsupported group size" (gemm_s4_f16.cu:119,233).
+ * Requires k % 128 == 0 (weight tiles are 128 rows whatever the group size), n_out % 16 == 0, tokens >= 0; A and X aligned to 16
  * bytes, Q to 4, C and R to 4 (to 8 when an MFMA prefill kernel runs, i.e. above 32 tokens, except
  * for W4A16_FUSED_SILU_FFN).
  * Numerics: the kernels for up to 32 tokens (and narrow matrices up to ~128) scale each group's
@@ -209,7 +214,8 @@ int w4a16_algo_count(void);
  *   A_dst  uint32 [k*m/8]  weights in the gfx950 tiled layout (same byte count as A_src)
  *   Q_dst  half2  [k/group_size, m] = (64 + zero, scale), bit-identical to the reference's
  * `workspace` (k/group_size*m halves) is accepted for signature compatibility and unused.
- * m = output features, must be a multiple of 16; k a multiple of 128. */
+ * m = output features, must be a multiple of 16; k a multiple of 128; group_size 128, 64 or 32 (the weight
+ * layout does not depend on it, Q has k / group_size rows). */
 int w4a16_convert_s4_k_m8(uint32_t* A_dst, void* Q_dst, void* workspace, const uint32_t* A_src,
                           const void* scales, const uint32_t* qzeros, int m, int k, int group_size,
                           void* stream);
@@ -217,10 +223,10 @@ int w4a16_convert_s4_k_m8(uint32_t* A_dst, void* Q_dst, void* workspace, const u
 /* The fused q|k|v matrix of a decoder layer, straight from the three AWQ tensors of the checkpoint:
  * what deploy_awq does with transpose_qk_s4 on q and k (lmdeploy/serve/turbomind/deploy.py:633-639;
  * scales by `permute`, :371-383), merge_qkv (:251-260) and convert_s4 (:660-670), in one gather.
- * qweight[i] uint32 [k, n_i/8], qzeros[i] uint32 [k/128, n_i/8], scales[i] fp16 [k/128, n_i] for
+ * qweight[i] uint32 [k, n_i/8], qzeros[i] uint32 [k/group_size, n_i/8], scales[i] fp16 [k/group_size, n_i] for
  * i = q, k, v with n = n_q, n_kv, n_kv.  Within every head of size_per_head columns of q and k,
  * output column 2i + r is source column r * size_per_head/2 + i.  A_dst: k * (n_q + 2 n_kv) / 2
- * bytes, Q_dst: half2 [k/128, n_q + 2 n_kv]. */
+ * bytes, Q_dst: half2 [k/group_size, n_q + 2 n_kv]. */
 int w4a16_deploy_qkv(uint32_t* A_dst, void* Q_dst, const uint32_t* const qweight[3], const uint32_t* const qzeros[3],
                      const void* const scales[3], int n_q, int n_kv, int k, int size_per_head, int group_size,
                      void* stream);
@@ -228,7 +234,7 @@ int w4a16_deploy_qkv(uint32_t* A_dst, void* Q_dst, const uint32_t* const qweight
 /* The fused gate|up matrix (w13) from the AWQ tensors of gate_proj (w1) and up_proj (w3): what
  * deploy_awq does with fuse_w1_w3_s4 (deploy.py:641-658: output column 2j = w1 column j, 2j + 1 =
  * w3 column j, for weights, zeros and scales) and convert_s4 (:660-670), in one gather.
- * A_dst: k * 2 * inter_size / 2 bytes, Q_dst: half2 [k/128, 2 * inter_size]. */
+ * A_dst: k * 2 * inter_size / 2 bytes, Q_dst: half2 [k/group_size, 2 * inter_size]. */
 int w4a16_deploy_w13(uint32_t* A_dst, void* Q_dst, const uint32_t* w1_qweight, const uint32_t* w3_qweight,
                      const uint32_t* w1_qzeros, const uint32_t* w3_qzeros, const void* w1_scales, const void* w3_scales,
                      int inter_size, int k, int group_size, void* stream);

@@ -42,6 +42,13 @@ bool aligned8(const void* p)
     return (reinterpret_cast<uintptr_t>(p) & 7u) == 0;
 }
 
+// Group sizes with kernels: the reference's 128 (gemm_s4_f16.cu:243-245 instantiates nothing else and leaves a
+// "TODO: add more group sizes"), plus 64 and 32.  Anything else gets the reference's error (gemm_s4_f16.cu:119).
+bool group_ok(int group_size)
+{
+    return group_size == 128 || group_size == 64 || group_size == 32;
+}
+
 }  // namespace
 
 struct w4a16_handle {
@@ -238,7 +245,7 @@ namespace {
 int check_gemm_args(const void* C, const void* A, const void* X, const void* Q, const void* R, int n_out, int tokens,
                     int k, int group_size, int epilogue)
 {
-    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
+    if (!group_ok(group_size)) return fail(W4A16_EGROUP, "unsupported group size");
     if (epilogue < W4A16_GEMM || epilogue > W4A16_FUSED_ADD) return fail(W4A16_EARG, "unknown epilogue %d", epilogue);
     if (n_out < 0 || tokens < 0 || k < 0) return fail(W4A16_EARG, "negative size");
     if (tokens == 0 || n_out == 0) return 1;  // nothing to do
@@ -427,11 +434,32 @@ int w4a16_algo_count(void)
 struct GemmPlan {
     int     algo;
     Scratch sc;
+    int     nq;  // quantisation groups per 128-row weight tile: 1 = the kernel table, 2 or 4 = the kernel for group size 64 / 32
 };
 
-int plan_gemm(w4a16_handle* h, const void* C, const void* R, int n_out, int tokens, int k, int epilogue, int algo_id,
-              hipStream_t st, GemmPlan* out)
+// Group sizes 64 and 32 have one kernel (strips, gemm_strip.hip): nothing to choose, no scratch.
+int plan_small_groups(int n_out, int tokens, int k, int group_size, int algo_id, GemmPlan* out)
 {
+    if (algo_id >= 0)
+        return fail(W4A16_EALGO, "kernel ids belong to group size 128; group size %d takes algo_id < 0 only", group_size);
+    const int nq = 128 / group_size;
+    if (!strip_groups_feasible(nq, n_out, tokens, k)) return fail(W4A16_ESHAPE, "no feasible kernel found");
+    out->algo = -1;
+    out->sc   = Scratch{};
+    out->nq   = nq;
+    return W4A16_OK;
+}
+
+hipError_t launch_plan(const GemmPlan& plan, const GemmArgs& g, hipStream_t st)
+{
+    return plan.nq > 1 ? strip_groups_launch(plan.nq, g, st) : algo_launch(plan.algo, g, plan.sc, st);
+}
+
+int plan_gemm(w4a16_handle* h, const void* C, const void* R, int n_out, int tokens, int k, int group_size, int epilogue,
+              int algo_id, hipStream_t st, GemmPlan* out)
+{
+    if (group_size != 128) return plan_small_groups(n_out, tokens, k, group_size, algo_id, out);
+    out->nq = 1;
     if (algo_id >= algo_count()) return fail(W4A16_EALGO, "algo_id %d out of range (0..%d)", algo_id, algo_count() - 1);
     const bool chosen = algo_id >= 0;
     if (!chosen) algo_id = pick_for(h, n_out, tokens, k);
@@ -467,10 +495,10 @@ int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const voi
     if (algo_id >= algo_count()) return fail(W4A16_EALGO, "algo_id %d out of range (0..%d)", algo_id, algo_count() - 1);
     if (int rc = check_device(h)) return rc;
     GemmPlan plan{};
-    if (int rc = plan_gemm(h, C, R, n_out, tokens, k, epilogue, algo_id, (hipStream_t)stream, &plan)) return rc;
+    if (int rc = plan_gemm(h, C, R, n_out, tokens, k, group_size, epilogue, algo_id, (hipStream_t)stream, &plan)) return rc;
     GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
                n_out,        tokens,             k,                  epilogue};
-    const hipError_t e = algo_launch(plan.algo, g, plan.sc, (hipStream_t)stream);
+    const hipError_t e = launch_plan(plan, g, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "w4a16_gemm launch");
     return W4A16_OK;
 }
@@ -482,6 +510,14 @@ int w4a16_gemm_static(void* C, const void* A, const void* X, const void* Q, cons
     if (chk < 0) return chk;
     if (chk > 0) return W4A16_OK;
     if (algo_id >= algo_count()) return fail(W4A16_EALGO, "algo_id %d out of range (0..%d)", algo_id, algo_count() - 1);
+    if (group_size != 128) {  // one kernel, no scratch at all
+        GemmPlan plan{};
+        if (int rc = plan_small_groups(n_out, tokens, k, group_size, algo_id, &plan)) return rc;
+        GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
+                   n_out,        tokens,             k,                  epilogue};
+        const hipError_t e = launch_plan(plan, g, (hipStream_t)stream);
+        return e == hipSuccess ? W4A16_OK : hip_fail(e, "w4a16_gemm_static launch");
+    }
     Scratch sc{};
     if (const hipError_t e = static_scratch(&sc); e != hipSuccess) return hip_fail(e, "w4a16_gemm_static set-up");
     if (algo_id < 0) algo_id = algo_pick(n_out, tokens, k, sc);
@@ -525,19 +561,20 @@ int w4a16_gemm_sequence(w4a16_handle* h, const w4a16_gemm_desc* gemms, int count
     }
     if (tokens == 0 || count == 0) return W4A16_OK;
     if (int rc = check_device(h)) return rc;
-    if (!(flags & W4A16_SEQ_PERSISTENT) || tokens > 16 || count == 1) {
+    if (!(flags & W4A16_SEQ_PERSISTENT) || tokens > 16 || count == 1 || group_size != 128) {
         // One launch per GEMM; stream order gives the dependencies.  Every GEMM is planned (kernel, workspace,
         // alignment) before the first one is launched: a list that cannot run as a whole runs not at all.
         std::vector<GemmPlan> plans(count);
         for (int i = 0; i < count; ++i) {
             const w4a16_gemm_desc& d = gemms[i];
-            if (int rc = plan_gemm(h, d.C, d.R, d.n_out, tokens, d.k, d.epilogue, -1, (hipStream_t)stream, &plans[i])) return rc;
+            if (int rc = plan_gemm(h, d.C, d.R, d.n_out, tokens, d.k, group_size, d.epilogue, -1, (hipStream_t)stream, &plans[i]))
+                return rc;
         }
         for (int i = 0; i < count; ++i) {
             const w4a16_gemm_desc& d = gemms[i];
             GemmArgs g{(uint16_t*)d.C, (const uint32_t*)d.A, (const uint16_t*)d.X, (const uint32_t*)d.Q, (const uint16_t*)d.R,
                        d.n_out,        tokens,                d.k,                  d.epilogue};
-            const hipError_t e = algo_launch(plans[i].algo, g, plans[i].sc, (hipStream_t)stream);
+            const hipError_t e = launch_plan(plans[i], g, (hipStream_t)stream);
             if (e != hipSuccess) return hip_fail(e, "w4a16_gemm_sequence launch");  // (the launch itself: earlier GEMMs are enqueued)
         }
         return W4A16_OK;
@@ -600,6 +637,7 @@ int w4a16_measure(w4a16_handle* h, void* C, const void* A, const void* X, const 
     if (!h) return fail(W4A16_EARG, "null handle");
     const int chk = check_gemm_args(C, A, X, Q, R, n_out, tokens, k, group_size, epilogue);
     if (chk < 0) return chk;
+    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");  // (64 and 32 have one kernel: nothing to measure)
     if (!metrics || capacity <= 0) return fail(W4A16_EARG, "no room for metrics");
     if (chk > 0) return 0;
     if (int rc = check_device(h)) return rc;
@@ -662,19 +700,19 @@ int w4a16_convert_s4_k_m8(uint32_t* A_dst, void* Q_dst, void* workspace, const u
                           const uint32_t* qzeros, int m, int k, int group_size, void* stream)
 {
     (void)workspace;
-    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
+    if (!group_ok(group_size)) return fail(W4A16_EGROUP, "unsupported group size");
     if (int c = check_repack("convert_s4_k_m8", m, k, 16, 128)) return c;
     if (m == 0 || k == 0) return W4A16_OK;
     if (!A_dst || !Q_dst || !A_src || !scales || !qzeros) return fail(W4A16_EARG, "convert_s4_k_m8: null pointer");
     const hipError_t e = launch_convert(A_dst, (uint32_t*)Q_dst, A_src, (const uint16_t*)scales, qzeros, m, k,
-                                        (hipStream_t)stream);
+                                        group_size, (hipStream_t)stream);
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "convert_s4_k_m8");
 }
 
 int w4a16_deploy_qkv(uint32_t* A_dst, void* Q_dst, const uint32_t* const qweight[3], const uint32_t* const qzeros[3],
                      const void* const scales[3], int n_q, int n_kv, int k, int size_per_head, int group_size, void* stream)
 {
-    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
+    if (!group_ok(group_size)) return fail(W4A16_EGROUP, "unsupported group size");
     if (n_q < 0 || n_kv < 0 || k < 0) return fail(W4A16_EARG, "deploy_qkv: negative size");
     if (size_per_head <= 0 || size_per_head % 2 != 0 || n_q % size_per_head != 0 || n_kv % size_per_head != 0)
         return fail(W4A16_ESHAPE, "deploy_qkv: q and k widths must be multiples of an even size_per_head");
@@ -689,7 +727,7 @@ int w4a16_deploy_qkv(uint32_t* A_dst, void* Q_dst, const uint32_t* const qweight
         if (width[i] > 0 && (!qweight[i] || !qzeros[i] || !scales[i])) return fail(W4A16_EARG, "deploy_qkv: null pointer");
         s[i] = (const uint16_t*)scales[i];
     }
-    const hipError_t e = launch_deploy(A_dst, (uint32_t*)Q_dst, qweight, qzeros, s, width, rotary, 0, k, (hipStream_t)stream);
+    const hipError_t e = launch_deploy(A_dst, (uint32_t*)Q_dst, qweight, qzeros, s, width, rotary, 0, k, group_size, (hipStream_t)stream);
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "deploy_qkv");
 }
 
@@ -697,7 +735,7 @@ int w4a16_deploy_w13(uint32_t* A_dst, void* Q_dst, const uint32_t* w1_qweight, c
                      const uint32_t* w1_qzeros, const uint32_t* w3_qzeros, const void* w1_scales, const void* w3_scales,
                      int inter_size, int k, int group_size, void* stream)
 {
-    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
+    if (!group_ok(group_size)) return fail(W4A16_EGROUP, "unsupported group size");
     if (inter_size < 0 || k < 0) return fail(W4A16_EARG, "deploy_w13: negative size");
     if (int c = check_repack("deploy_w13", inter_size, k, 8, 128)) return c;
     if (inter_size == 0 || k == 0) return W4A16_OK;
@@ -708,7 +746,7 @@ int w4a16_deploy_w13(uint32_t* A_dst, void* Q_dst, const uint32_t* w1_qweight, c
     const uint16_t* s[3]      = {(const uint16_t*)w1_scales, (const uint16_t*)w3_scales, nullptr};
     const int       width[3]  = {inter_size, inter_size, 0};
     const int       rotary[3] = {0, 0, 0};
-    const hipError_t e = launch_deploy(A_dst, (uint32_t*)Q_dst, qw, qz, s, width, rotary, 1, k, (hipStream_t)stream);
+    const hipError_t e = launch_deploy(A_dst, (uint32_t*)Q_dst, qw, qz, s, width, rotary, 1, k, group_size, (hipStream_t)stream);
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "deploy_w13");
 }
 
@@ -717,7 +755,7 @@ int w4a16_reformat_s4_k_m8(uint32_t* dst, const uint32_t* src, int m, int k, voi
     if (int c = check_repack("reformat_s4_k_m8", m, k, 16, 128)) return c;
     if (m == 0 || k == 0) return W4A16_OK;
     if (!dst || !src) return fail(W4A16_EARG, "reformat_s4_k_m8: null pointer");
-    const hipError_t e = launch_convert(dst, nullptr, src, nullptr, nullptr, m, k, (hipStream_t)stream);
+    const hipError_t e = launch_convert(dst, nullptr, src, nullptr, nullptr, m, k, 128, (hipStream_t)stream);
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "reformat_s4_k_m8");
 }
 
@@ -753,22 +791,22 @@ int w4a16_dequantize_s4(void* dst, const uint32_t* src, size_t count, void* stre
 int w4a16_unpack_repacked(uint32_t* qweight, uint32_t* qzeros, void* scales, const uint32_t* A, const void* Q, int m,
                           int k, int group_size, void* stream)
 {
-    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
+    if (!group_ok(group_size)) return fail(W4A16_EGROUP, "unsupported group size");
     if (int c = check_repack("unpack_repacked", m, k, 16, 128)) return c;
     if (m == 0 || k == 0) return W4A16_OK;
     if ((qweight && !A) || ((qzeros || scales) && !Q)) return fail(W4A16_EARG, "unpack_repacked: null pointer");
     const hipError_t e = launch_unpack(qweight, qzeros, (uint16_t*)scales, A, (const uint32_t*)Q, m, k,
-                                       (hipStream_t)stream);
+                                       group_size, (hipStream_t)stream);
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "unpack_repacked");
 }
 
 int w4a16_dequantize_repacked(void* W, const uint32_t* A, const void* Q, int m, int k, int group_size, void* stream)
 {
-    if (group_size != 128) return fail(W4A16_EGROUP, "unsupported group size");
+    if (!group_ok(group_size)) return fail(W4A16_EGROUP, "unsupported group size");
     if (int c = check_repack("dequantize_repacked", m, k, 16, 128)) return c;
     if (m == 0 || k == 0) return W4A16_OK;
     if (!W || !A || !Q) return fail(W4A16_EARG, "dequantize_repacked: null pointer");
-    const hipError_t e = launch_dequantize_repacked((uint16_t*)W, A, (const uint32_t*)Q, m, k, (hipStream_t)stream);
+    const hipError_t e = launch_dequantize_repacked((uint16_t*)W, A, (const uint32_t*)Q, m, k, group_size, (hipStream_t)stream);
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "dequantize_repacked");
 }
 

@@ -55,6 +55,42 @@ __global__ void __launch_bounds__(64 * kWaves) strip_kernel(const StripParams p)
     }
 }
 
+// The same kernel for group sizes 64 and 32 (NQ = 2, 4 quantisation groups per 128-row tile): 16 token rows per
+// workgroup whatever the token count, the epilogue chosen at run time, strips of at most kMaxRQ tiles (a tile
+// brings NQ scale words along) - eight instantiations instead of ninety-six.
+constexpr int kMaxRQ = 4;
+template<int RMAX, int NQ>
+__global__ void __launch_bounds__(64 * kWaves) strip_kernel_q(const StripParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) u32x4_t smem[];
+    for (int pass = 0; pass < p.passes; ++pass) {
+        const int  bx   = pass * gridDim.x + blockIdx.x;
+        const bool wide = bx < p.rem;
+        const int  col0 = bx * p.base + min(bx, p.rem);
+        if (pass) __syncthreads();
+        bool done = false;
+        if constexpr (RMAX > 1) {
+            if (!wide && p.base == RMAX - 1) {
+                strip_body<RMAX - 1, 16, kEpiRuntime, false, kWaves, NoWait, NQ>(p, col0, smem);
+                done = true;
+            }
+        }
+        if (!done) strip_body<RMAX, 16, kEpiRuntime, false, kWaves, NoWait, NQ>(p, col0, smem);
+    }
+}
+
+template<int NQ>
+hipError_t launch_q(int rmax, const StripParams& p, dim3 grid, size_t lds, hipStream_t st)
+{
+    const dim3 block(64 * kWaves);
+    switch (rmax) {
+        case 1: return launch_kernel(strip_kernel_q<1, NQ>, grid, block, lds, st, p);
+        case 2: return launch_kernel(strip_kernel_q<2, NQ>, grid, block, lds, st, p);
+        case 3: return launch_kernel(strip_kernel_q<3, NQ>, grid, block, lds, st, p);
+        default: return launch_kernel(strip_kernel_q<4, NQ>, grid, block, lds, st, p);
+    }
+}
+
 template<int RMAX, int TP>
 hipError_t launch_rt(const StripParams& p, dim3 grid, size_t lds, int epilogue, hipStream_t st)
 {
@@ -99,14 +135,14 @@ constexpr int kInPasses = 3;  // value of `per_cu` that asks for one workgroup p
 
 // `per_cu` strips per CU are aimed for; more if a strip would otherwise be wider than the limit.
 // block_t = tokens per workgroup: 16 (activation rows padded down to 4 or 8 for fewer tokens) or 32.
-StripPlan make_plan(int per_cu, int block_t, int N, int T, int K)
+StripPlan make_plan(int per_cu, int block_t, int N, int T, int K, int maxr_limit = kMaxR)
 {
     StripPlan pl{};
     if (N <= 0 || K <= 0 || T <= 0 || N % kTileN != 0 || K % kGroup != 0 || per_cu < 1) return pl;
     if (block_t != 16 && block_t != 32) return pl;
     if (block_t == 32 && T <= 16) return pl;  // the 16-token kernel covers these
     const int NT   = N / kTileN;
-    const int maxr = block_t == 32 ? kMaxR32 : kMaxR;
+    const int maxr = std::min(maxr_limit, block_t == 32 ? kMaxR32 : kMaxR);
     int       m    = per_cu == kInPasses ? 1 : per_cu;
     while ((NT + kNumCU * m - 1) / (kNumCU * m) > maxr) ++m;
     pl.strips = std::min(NT, kNumCU * m);
@@ -167,6 +203,24 @@ hipError_t strip_launch(int per_cu, int block_t, const GemmArgs& a, hipStream_t 
         case 7: return launch_r<7>(tp, p, grid, lds, a.epilogue, st);
         default: return launch_r<8>(tp, p, grid, lds, a.epilogue, st);
     }
+}
+
+// Group sizes 64 and 32: strips of up to kMaxRQ tiles, one workgroup per strip (as many workgroups per CU as that
+// takes), token blocks of 16 side by side in the grid for more than 16 tokens (each block streams the weights again).
+bool strip_groups_feasible(int nq, int N, int T, int K)
+{
+    return (nq == 2 || nq == 4) && make_plan(1, 16, N, T, K, kMaxRQ).ok;
+}
+
+hipError_t strip_groups_launch(int nq, const GemmArgs& a, hipStream_t st)
+{
+    const StripPlan pl = make_plan(1, 16, a.N, a.T, a.K, kMaxRQ);
+    if (!pl.ok || (nq != 2 && nq != 4)) return hipErrorInvalidValue;
+    StripParams  p{a.C, reinterpret_cast<const u32x4_t*>(a.A), a.X, a.Q, a.R, a.N, a.T, a.K, pl.base, pl.rem,
+                   a.epilogue, pl.passes};
+    const dim3   grid(pl.strips, (a.T + 15) / 16);
+    const size_t lds = (size_t)kWaves * std::max(pl.rmax * 1024, 16 * 256);
+    return nq == 2 ? launch_q<2>(pl.rmax, p, grid, lds, st) : launch_q<4>(pl.rmax, p, grid, lds, st);
 }
 
 }  // namespace w4a16

@@ -171,7 +171,7 @@ split_q_kernel(uint32_t* __restrict__ qzeros, uint16_t* __restrict__ scales, con
 // W[k, n] = mul.ftz(sub(64 + q, 64 + z), s): one thread per repacked word (8 rows of a column)
 __global__ void __launch_bounds__(kThreads)
 dequantize_repacked_kernel(uint16_t* __restrict__ W, const uint32_t* __restrict__ A,
-                           const uint32_t* __restrict__ Q, int N, int K)
+                           const uint32_t* __restrict__ Q, int N, int K, int group)
 {
     const int64_t w     = global_id();
     const int64_t words = (int64_t)N * K / 8;
@@ -186,7 +186,7 @@ dequantize_repacked_kernel(uint16_t* __restrict__ W, const uint32_t* __restrict_
     const int     k0   = kt * kGroup + 32 * j + 8 * (lane >> 4);
     half2_t       z1024, z64;
     half_t        s;
-    split_q(Q[(int64_t)kt * N + n], z1024, z64, s);
+    split_q(Q[(int64_t)(k0 / group) * N + n], z1024, z64, s);  // (a word's 8 rows never straddle two groups: group >= 32)
     // flush a subnormal scale first, as the .ftz multiply of the reference reads it
     uint16_t sb = __builtin_bit_cast(uint16_t, s);
     if ((sb & 0x7c00u) == 0) sb &= 0x8000u;
@@ -297,10 +297,10 @@ inline unsigned blocks_for(int64_t n)
 }  // namespace
 
 hipError_t launch_convert(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* A_src, const uint16_t* scales,
-                          const uint32_t* qzeros, int m, int k, hipStream_t st)
+                          const uint32_t* qzeros, int m, int k, int group, hipStream_t st)
 {
     const int64_t words = (int64_t)m * k / 8;
-    const int64_t qn    = (int64_t)(k / kGroup) * m;
+    const int64_t qn    = (int64_t)(k / group) * m;
     if (words == 0) return hipSuccess;
     hipError_t e = hipSuccess;
     if (A_dst) e = launch_kernel(repack_weights_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, A_dst, A_src, m, k);
@@ -311,7 +311,7 @@ hipError_t launch_convert(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* A_sr
 
 hipError_t launch_deploy(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* const qw[3], const uint32_t* const qz[3],
                          const uint16_t* const s[3], const int width[3], const int rotary[3], int interleave, int k,
-                         hipStream_t st)
+                         int group, hipStream_t st)
 {
     ColumnSource cs{};
     int          m = 0;
@@ -322,19 +322,19 @@ hipError_t launch_deploy(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* const
     }
     cs.interleave       = interleave;
     const int64_t words = (int64_t)m * k / 8;
-    const int64_t qn    = (int64_t)(k / kGroup) * m;
+    const int64_t qn    = (int64_t)(k / group) * m;
     if (words == 0) return hipSuccess;
     hipError_t e = launch_kernel(deploy_weights_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, A_dst, cs, m, k);
     if (e == hipSuccess)
-        e = launch_kernel(deploy_q_kernel, dim3(blocks_for(qn)), dim3(kThreads), 0, st, Q_dst, cs, m, k / kGroup);
+        e = launch_kernel(deploy_q_kernel, dim3(blocks_for(qn)), dim3(kThreads), 0, st, Q_dst, cs, m, k / group);
     return e;
 }
 
 hipError_t launch_unpack(uint32_t* qweight, uint32_t* qzeros, uint16_t* scales, const uint32_t* A,
-                         const uint32_t* Q, int m, int k, hipStream_t st)
+                         const uint32_t* Q, int m, int k, int group, hipStream_t st)
 {
     const int64_t words = (int64_t)m * k / 8;
-    const int64_t qw    = (int64_t)(k / kGroup) * m / 8;
+    const int64_t qw    = (int64_t)(k / group) * m / 8;
     if (words == 0) return hipSuccess;
     hipError_t e = hipSuccess;
     if (qweight) e = launch_kernel(unrepack_weights_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, qweight, A, m, k);
@@ -343,12 +343,12 @@ hipError_t launch_unpack(uint32_t* qweight, uint32_t* qzeros, uint16_t* scales, 
     return e;
 }
 
-hipError_t launch_dequantize_repacked(uint16_t* W, const uint32_t* A, const uint32_t* Q, int m, int k,
+hipError_t launch_dequantize_repacked(uint16_t* W, const uint32_t* A, const uint32_t* Q, int m, int k, int group,
                                       hipStream_t st)
 {
     const int64_t words = (int64_t)m * k / 8;
     if (words == 0) return hipSuccess;
-    return launch_kernel(dequantize_repacked_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, W, A, Q, m, k);
+    return launch_kernel(dequantize_repacked_kernel, dim3(blocks_for(words)), dim3(kThreads), 0, st, W, A, Q, m, k, group);
 }
 
 hipError_t launch_dequantize_s4(void* dst, const uint32_t* src, size_t count, hipStream_t st)

@@ -120,10 +120,11 @@ __device__ __forceinline__ void static_for(F&& f)
 
 // Everything one wave holds for one group: R weight tiles, their Q words, and the activations of
 // the group (NX loads of four token rows x 256 bytes each, one 16-byte chunk per lane).
-template<int R, int NX>
+// NQ = quantisation groups per weight tile: 1 (group size 128), 2 (64) or 4 (32); tile r's words are q[r * NQ ..].
+template<int R, int NX, int NQ = 1>
 struct Stage {
     u32x4_t  w[R];
-    uint32_t q[R];
+    uint32_t q[R * NQ];
     u32x4_t  x[NX > 0 ? NX : 1];  // (NX = 0: the activations go straight to LDS)
 };
 
@@ -138,7 +139,10 @@ struct NoWait {
     __device__ __forceinline__ void operator()() const {}
 };
 // NW = waves of the workgroup = slices of K.
-template<int R, int TP, int EPI, bool SEQ = false, int NW = kWaves, typename Ready = NoWait>
+// NQ: quantisation groups per 128-row weight tile (group sizes 128, 64, 32 = NQ 1, 2, 4).  The weight layout does
+// not depend on it; Q then has NQ rows per tile row, and every 128 / NQ rows of a tile have their own scale and
+// zero point: NQ shorter MFMA chains per tile, each scaled into the accumulator by itself.
+template<int R, int TP, int EPI, bool SEQ = false, int NW = kWaves, typename Ready = NoWait, int NQ = 1>
 __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4_t* smem, Ready&& inputs_ready = Ready{})
 {
     const int tid  = threadIdx.x;
@@ -205,7 +209,8 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     const char* Xb = reinterpret_cast<const char*>(p.X);
 
     // All loads of group g into stage s (number d); enable = false turns them into no-ops that still count.
-    using StageT = Stage<R, NXR>;
+    using StageT = Stage<R, NXR, NQ>;
+    static_assert(NQ == 1 || NQ == 2 || NQ == 4, "group sizes 128, 64 and 32");
     auto issue_x = [&](StageT& s, int d, int g, bool enable) {
         const int flag = __builtin_amdgcn_readfirstlane(enable ? 1 : 0);
         static_for<0, NX>([&](auto i) {
@@ -216,8 +221,10 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     };
     auto issue_wq = [&](StageT& s, int g, bool enable) {
         const int flag = __builtin_amdgcn_readfirstlane(enable ? 1 : 0);
-        const char* qg = Qb + (int64_t)g * N * 4;
-        static_for<0, R>([&](auto r) { mload32<r * 64>(s.q[r], q_off, qg, flag); });
+        static_for<0, NQ>([&](auto sub) {
+            const char* qg = Qb + ((int64_t)g * NQ + sub) * N * 4;
+            static_for<0, R>([&](auto r) { mload32<r * 64>(s.q[r * NQ + sub], q_off, qg, flag); });
+        });
         // the tiles of a group are contiguous; immediates reach 4 KiB, so every fourth tile gets a new base
         static_for<0, R>([&](auto r) {
             const char* wg = Ab + ((int64_t)g * NT + (r / 4) * 4) * 1024;
@@ -228,7 +235,7 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
         issue_x(s, d, g, enable);
         issue_wq(s, g, enable);
     };
-    constexpr int kLoads = 2 * R + NX;  // loads per stage
+    constexpr int kLoads = R + R * NQ + NX;  // loads per stage
 
     const UnpackConsts uc;
     float4_t           acc[H][R];
@@ -269,56 +276,61 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
         constexpr int U = 2;
 #pragma unroll
         for (int r0 = 0; r0 < R; r0 += U) {
-            float4_t g4[H][U];
-            float    sf[U];
-            half8_t  bz[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int r = r0 + u < R ? r0 + u : R - 1;
-                // B operand that removes the unpack offsets and the zero point: -(1024 + z) under
-                // the low-nibble pairs, -(64 + z) under the high-nibble pairs
-                const half2_t  h2  = as_half2(s.q[r]);
-                const half2_t  n64 = half2_t{h2[0], h2[0]} * half2_t{(half_t)-1.f, (half_t)-1.f};
-                const uint32_t zb  = ((s.q[r] >> 4) & 0xfu) * 0x10001u + 0xE400E400u;  // -(1024 + z) twice
-                bz[u][0] = as_half2(zb)[0]; bz[u][1] = as_half2(zb)[1]; bz[u][2] = n64[0]; bz[u][3] = n64[1];
-                bz[u][4] = bz[u][0]; bz[u][5] = bz[u][1]; bz[u][6] = bz[u][2]; bz[u][7] = bz[u][3];
-                // Convert the scale now and hide it from the optimiser: otherwise the conversion is
-                // folded into the final multiply-add, the Q word stays live past the refill of this
-                // stage, and the refill lands in a copy that is moved back while still in flight.
-                sf[u] = scale_is_normal(s.q[r]) ? (float)h2[1] : 0.f;
-                asm volatile("" : "+v"(sf[u]));
+            for (int sub = 0; sub < NQ; ++sub) {  // the rows of the tile that share a scale and a zero point
+                constexpr int JN = 4 / NQ;        // k32 chunks per quantisation group
+                float4_t g4[H][U];
+                float    sf[U];
+                half8_t  bz[U];
 #pragma unroll
-                for (int h = 0; h < H; ++h) g4[h][u] = float4_t{0.f, 0.f, 0.f, 0.f};
-            }
+                for (int u = 0; u < U; ++u) {
+                    const int      r  = r0 + u < R ? r0 + u : R - 1;
+                    const uint32_t qw = s.q[r * NQ + sub];
+                    // B operand that removes the unpack offsets and the zero point: -(1024 + z) under
+                    // the low-nibble pairs, -(64 + z) under the high-nibble pairs
+                    const half2_t  h2  = as_half2(qw);
+                    const half2_t  n64 = half2_t{h2[0], h2[0]} * half2_t{(half_t)-1.f, (half_t)-1.f};
+                    const uint32_t zb  = ((qw >> 4) & 0xfu) * 0x10001u + 0xE400E400u;  // -(1024 + z) twice
+                    bz[u][0] = as_half2(zb)[0]; bz[u][1] = as_half2(zb)[1]; bz[u][2] = n64[0]; bz[u][3] = n64[1];
+                    bz[u][4] = bz[u][0]; bz[u][5] = bz[u][1]; bz[u][6] = bz[u][2]; bz[u][7] = bz[u][3];
+                    // Convert the scale now and hide it from the optimiser: otherwise the conversion is
+                    // folded into the final multiply-add, the Q word stays live past the refill of this
+                    // stage, and the refill lands in a copy that is moved back while still in flight.
+                    sf[u] = scale_is_normal(qw) ? (float)h2[1] : 0.f;
+                    asm volatile("" : "+v"(sf[u]));
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+                    for (int h = 0; h < H; ++h) g4[h][u] = float4_t{0.f, 0.f, 0.f, 0.f};
+                }
+#pragma unroll
+                for (int j = sub * JN; j < (sub + 1) * JN; ++j) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+#pragma unroll
+                        for (int h = 0; h < H; ++h)
+                            if (r0 + u < R) g4[h][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[h][j], bz[u], g4[h][u], 0, 0, 0);
+                }
+#pragma unroll
+                for (int j = sub * JN; j < (sub + 1) * JN; ++j) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        if (r0 + u < R) {
+                            uint32_t v[4];
+                            unpack_offset(s.w[r0 + u][j], v, uc);
+                            half8_t wf;
+                            wf[0] = as_half2(v[0])[0]; wf[1] = as_half2(v[0])[1]; wf[2] = as_half2(v[1])[0]; wf[3] = as_half2(v[1])[1];
+                            wf[4] = as_half2(v[2])[0]; wf[5] = as_half2(v[2])[1]; wf[6] = as_half2(v[3])[0]; wf[7] = as_half2(v[3])[1];
+#pragma unroll
+                            for (int h = 0; h < H; ++h)
+                                g4[h][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[h][j], wf, g4[h][u], 0, 0, 0);
+                        }
+                    }
+                }
 #pragma unroll
                 for (int u = 0; u < U; ++u)
 #pragma unroll
                     for (int h = 0; h < H; ++h)
-                        if (r0 + u < R) g4[h][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[h][j], bz[u], g4[h][u], 0, 0, 0);
+                        if (r0 + u < R) acc[h][r0 + u] += sf[u] * g4[h][u];
             }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    if (r0 + u < R) {
-                        uint32_t v[4];
-                        unpack_offset(s.w[r0 + u][j], v, uc);
-                        half8_t wf;
-                        wf[0] = as_half2(v[0])[0]; wf[1] = as_half2(v[0])[1]; wf[2] = as_half2(v[1])[0]; wf[3] = as_half2(v[1])[1];
-                        wf[4] = as_half2(v[2])[0]; wf[5] = as_half2(v[2])[1]; wf[6] = as_half2(v[3])[0]; wf[7] = as_half2(v[3])[1];
-#pragma unroll
-                        for (int h = 0; h < H; ++h)
-                            g4[h][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[h][j], wf, g4[h][u], 0, 0, 0);
-                    }
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-#pragma unroll
-                for (int h = 0; h < H; ++h)
-                    if (r0 + u < R) acc[h][r0 + u] += sf[u] * g4[h][u];
         }
     };
     // Wait until the stage's loads are complete (loads return in order: at most `kLoads` younger
@@ -326,7 +338,9 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     // the wait.
     auto pin = [&](StageT& s) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) asm volatile("" : "+v"(s.w[r]), "+v"(s.q[r]));
+        for (int r = 0; r < R; ++r) asm volatile("" : "+v"(s.w[r]));
+#pragma unroll
+        for (int r = 0; r < R * NQ; ++r) asm volatile("" : "+v"(s.q[r]));
 #pragma unroll
         for (int i = 0; i < NXR; ++i) asm volatile("" : "+v"(s.x[i]));
     };
@@ -337,10 +351,9 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
 #pragma unroll
     for (int d = 0; d < D; ++d) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            st[d].w[r] = u32x4_t{0, 0, 0, 0};
-            st[d].q[r] = 0;
-        }
+        for (int r = 0; r < R; ++r) st[d].w[r] = u32x4_t{0, 0, 0, 0};
+#pragma unroll
+        for (int r = 0; r < R * NQ; ++r) st[d].q[r] = 0;
 #pragma unroll
         for (int i = 0; i < NXR; ++i) st[d].x[i] = u32x4_t{0, 0, 0, 0};
     }

@@ -100,14 +100,14 @@ hipError_t static_scratch(Scratch* out);
 hipError_t clear_counters(const Scratch& sc, int n, hipStream_t st);
 
 hipError_t launch_convert(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* A_src, const uint16_t* scales,
-                          const uint32_t* qzeros, int m, int k, hipStream_t st);
+                          const uint32_t* qzeros, int m, int k, int group, hipStream_t st);
 // up to three AWQ tensors -> one deployable (A, Q): side by side, or (interleave) gate/up column pairs
 hipError_t launch_deploy(uint32_t* A_dst, uint32_t* Q_dst, const uint32_t* const qw[3], const uint32_t* const qz[3],
                          const uint16_t* const s[3], const int width[3], const int rotary[3], int interleave, int k,
-                         hipStream_t st);
+                         int group, hipStream_t st);
 hipError_t launch_unpack(uint32_t* qweight, uint32_t* qzeros, uint16_t* scales, const uint32_t* A,
-                         const uint32_t* Q, int m, int k, hipStream_t st);
-hipError_t launch_dequantize_repacked(uint16_t* W, const uint32_t* A, const uint32_t* Q, int m, int k,
+                         const uint32_t* Q, int m, int k, int group, hipStream_t st);
+hipError_t launch_dequantize_repacked(uint16_t* W, const uint32_t* A, const uint32_t* Q, int m, int k, int group,
                                       hipStream_t st);
 hipError_t launch_dequantize_s4(void* dst, const uint32_t* src, size_t count, hipStream_t st);
 hipError_t launch_fuse_w1_w3(uint32_t* dst, const uint32_t* src, int m, int k, hipStream_t st);
@@ -134,6 +134,9 @@ bool       strip_feasible(int per_cu, int block_t, int N, int T, int K);
 int        strip_grid(int per_cu, int block_t, int N, int T, int K);
 int        strip_width(int per_cu, int block_t, int N, int T, int K);  // column tiles of the widest strip
 hipError_t strip_launch(int per_cu, int block_t, const GemmArgs& a, hipStream_t st);
+// the strip kernel for group sizes 64 and 32 (nq = 2, 4 quantisation groups per 128-row weight tile), any token count
+bool       strip_groups_feasible(int nq, int N, int T, int K);
+hipError_t strip_groups_launch(int nq, const GemmArgs& a, hipStream_t st);
 
 // A sequence of decode GEMMs (up to 16 tokens) in one persistent launch (gemm_sequence.hip)
 struct SeqGemm {

@@ -82,7 +82,7 @@ def deploy_awq_weights(params: Mapping[str, torch.Tensor], num_layer: int, out_d
     if tp != 1:
         raise NotImplementedError("tensor-parallel export is not part of this one-GPU build: cut the tiled "
                                   "weights on 16-column / 128-row tile boundaries per rank")
-    if group_size != 128:
+    if group_size not in (128, 64, 32):
         raise ValueError("unsupported group size")
     wdir = os.path.join(out_dir, "weights")
     os.makedirs(wdir, exist_ok=True)

@@ -20,7 +20,7 @@ pytestmark = pytest.mark.gpu
 H, F, L, G = 256, 384, 2, 128   # hidden (2 heads of 128), intermediate, layers, group size
 
 
-def _awq(rng, K, N):
+def _awq(rng, K, N, G=G):
     q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
     z = rng.integers(0, 16, size=(K // G, N), dtype=np.uint8)
     s = (np.abs(rng.standard_normal((K // G, N))) * 0.01 + 1e-3).astype(np.float16)
@@ -127,7 +127,8 @@ def test_reference_written_workspace_loads_into_the_same_tensors(tmp_path):
         deploy.load_workspace_linear(str(wdir), "layers.0.attention.wo", K, N + 16)
 
 
-def test_fused_tensor_entry_points_equal_the_reference_steps_bit_for_bit():
+@pytest.mark.parametrize("G", [128, 64, 32])
+def test_fused_tensor_entry_points_equal_the_reference_steps_bit_for_bit(G):
     """`w4a16_deploy_qkv` / `w4a16_deploy_w13` against the oracle's restatement of the reference's separate
     steps (format.cu:115-130 on qweight and qzeros, deploy.py:371-383 and :651-652 on the scales, then
     convert_s4_k_m8), with grouped-query widths (k and v narrower than q) and several heads."""
@@ -141,8 +142,8 @@ def test_fused_tensor_entry_points_equal_the_reference_steps_bit_for_bit():
         return s.reshape(g, dim // D, 2, D // 2).transpose(0, 1, 3, 2).reshape(g, dim)
 
     for n_q, n_kv in ((1024, 256), (256, 256)):
-        q, k, v = _awq(rng, K, n_q), _awq(rng, K, n_kv), _awq(rng, K, n_kv)
-        A, Q = tm.deploy_qkv(tuple(map(dev, q)), tuple(map(dev, k)), tuple(map(dev, v)), D)
+        q, k, v = _awq(rng, K, n_q, G), _awq(rng, K, n_kv, G), _awq(rng, K, n_kv, G)
+        A, Q = tm.deploy_qkv(tuple(map(dev, q)), tuple(map(dev, k)), tuple(map(dev, v)), D, G)
         qw = np.concatenate([O.transpose_qk_s4_k_m8_hf(q[0], n_q, K, D), O.transpose_qk_s4_k_m8_hf(k[0], n_kv, K, D), v[0]], axis=1)
         qz = np.concatenate([O.transpose_qk_s4_k_m8_hf(q[1], n_q, K // G, D), O.transpose_qk_s4_k_m8_hf(k[1], n_kv, K // G, D),
                              v[1]], axis=1)
@@ -152,8 +153,8 @@ def test_fused_tensor_entry_points_equal_the_reference_steps_bit_for_bit():
         assert np.array_equal(A.cpu().numpy().view(np.uint32).reshape(-1), A_ref)
         assert np.array_equal(Q.cpu().numpy().view(np.uint32), Q_ref)
     F1 = 1408
-    w1, w3 = _awq(rng, K, F1), _awq(rng, K, F1)
-    A, Q = tm.deploy_w13(tuple(map(dev, w1)), tuple(map(dev, w3)))
+    w1, w3 = _awq(rng, K, F1, G), _awq(rng, K, F1, G)
+    A, Q = tm.deploy_w13(tuple(map(dev, w1)), tuple(map(dev, w3)), G)
     qw = O.fuse_w1_w3_s4_k_m8(np.concatenate([w1[0], w3[0]]), F1, K)
     qz = O.fuse_w1_w3_s4_k_m8(np.concatenate([w1[1], w3[1]]), F1, K // G)
     s = np.stack([w1[2], w3[2]], axis=-1).reshape(K // G, 2 * F1)      # deploy.py:651-652
@@ -161,4 +162,4 @@ def test_fused_tensor_entry_points_equal_the_reference_steps_bit_for_bit():
     assert np.array_equal(A.cpu().numpy().view(np.uint32).reshape(-1), A_ref)
     assert np.array_equal(Q.cpu().numpy().view(np.uint32), Q_ref)
     with pytest.raises(tm.W4A16Error):
-        tm.deploy_qkv(tuple(map(dev, q)), tuple(map(dev, k)), tuple(map(dev, v)), 96)     # 256 is not a multiple of 96
+        tm.deploy_qkv(tuple(map(dev, q)), tuple(map(dev, k)), tuple(map(dev, v)), 96, G)     # 256 is not a multiple of 96

@@ -612,7 +612,7 @@ def test_ffn_block(tm, gemm):
     want = O.gemm_s4_f16(g_host, d2["qweight"], d2["qzeros"], d2["scales"], 128, O.EPI_ADD, d2["R"])
     assert O.max_abs_rel(res.cpu().numpy(), want) <= TOL
     with pytest.raises(tm.W4A16Error):
-        gemm.ffn(out, gating, x, A13, Q13, A2, Q2, H, F, T, group_size=64)
+        gemm.ffn(out, gating, x, A13, Q13, A2, Q2, H, F, T, group_size=256)
 
 
 def test_errors(tm, gemm):
@@ -622,7 +622,7 @@ def test_errors(tm, gemm):
     X = dev(d["X"])
     C = torch.empty(T, N, dtype=torch.float16, device="cuda")
     with pytest.raises(tm.W4A16Error, match="unsupported group size") as e:
-        gemm.Run(C, A, X, Q, N, T, K, 64)
+        gemm.Run(C, A, X, Q, N, T, K, 256)
     assert e.value.code == -1
     with pytest.raises(tm.W4A16Error, match="no feasible kernel found") as e:
         gemm.Run(C, A, X, Q, N + 8, T, K, 128)
@@ -693,3 +693,94 @@ def test_measured_choices_survive_in_a_file(tm, tmp_path):
     lines = text.splitlines()
     open(other, "w").write("\n".join([lines[0], "72 4 256 0", lines[1]]) + "\n")
     assert g3.load_tuning(other) == 1 and g3.pick(N, T, K) == fastest
+
+
+# ------------------------------------------------------------------ group sizes 64 and 32
+@pytest.mark.parametrize("gs", [64, 32])
+def test_group_sizes_64_and_32_conversion_is_bit_exact(tm, gs):
+    """The weight layout does not depend on the group size; Q has K / gs rows.  Repack, Q, the inverse and the
+    dequantised weights, word for word against the oracle."""
+    K, N = 640, 256
+    d = O.make_inputs(6400 + gs, 1, K, N, gs)
+    qw, qz, s = dev(d["qweight"]), dev(d["qzeros"]), dev(d["scales"])
+    A, Q = torch.zeros_like(qw), torch.zeros_like(s, dtype=torch.int32)
+    tm.convert_s4_k_m8(A, Q, torch.zeros_like(s), qw, s, qz, N, K, gs)
+    A_ref, Q_ref = O.convert_s4_k_m8(d["qweight"], d["scales"], d["qzeros"], N, K, gs)
+    assert np.array_equal(host_u32(A).reshape(-1), A_ref)
+    assert np.array_equal(host_u32(Q), Q_ref)
+    qw2, qz2, s2 = tm.unpack_repacked(A, Q, N, K, gs)
+    assert torch.equal(qw2, qw) and torch.equal(qz2, qz) and torch.equal(s2.view(torch.int16), s.view(torch.int16))
+    W = tm.dequantize_repacked(A, Q, N, K, gs).cpu().numpy()
+    W_ref = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], gs)
+    assert np.array_equal(W.view(np.uint16), W_ref.view(np.uint16))
+
+
+@pytest.mark.parametrize("gs", [64, 32])
+@pytest.mark.parametrize("K,N", [(1024, 256), (640, 4096), (256, 22016), (384, 57344), (128, 48)])
+def test_group_sizes_64_and_32_gemm(tm, gemm, gs, K, N):
+    """One kernel family serves these group sizes (strips of up to four column tiles, the scale applied per
+    quantisation group inside the tile): narrow and wide matrices, uneven deals, one and several strips per CU,
+    token counts on both sides of the 16-token block, every epilogue, against the oracle."""
+    Ts = (1, 5, 16, 17, 40) if N > 8192 else (1, 5, 16, 17, 40, 130)
+    d = O.make_inputs(6500 + gs + N, max(Ts), K, N, gs, residual=True)
+    qw, qz, s = dev(d["qweight"]), dev(d["qzeros"]), dev(d["scales"])
+    A, Q = torch.zeros_like(qw), torch.zeros_like(s, dtype=torch.int32)
+    tm.convert_s4_k_m8(A, Q, torch.zeros_like(s), qw, s, qz, N, K, gs)
+    W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], gs)
+    for T in Ts:
+        X, R = dev(d["X"][:T]), dev(d["R"][:T])
+        acc = O.gemm_acc(d["X"][:T], W)
+        for kind in (0, 1, 2):
+            want = O.epilogue(acc, kind, d["R"][:T] if kind == 2 else None)
+            C = torch.full((T, N // 2 if kind == 1 else N), float("nan"), dtype=torch.float16, device="cuda")
+            gemm.Run(C, A, X, Q, N, T, K, gs, kind, -1, residual=R if kind == 2 else None)
+            torch.cuda.synchronize()
+            assert_close(C.cpu().numpy(), want, (gs, K, N, T, kind))
+            if T in (5, 40):   # the entry point without a handle runs the same kernel
+                Cs = torch.empty_like(C)
+                tm.gemm_static(Cs, A, X, Q, N, T, K, gs, kind, -1, residual=R if kind == 2 else None)
+                torch.cuda.synchronize()
+                assert torch.equal(Cs.view(torch.int16), C.view(torch.int16))
+
+
+def test_group_size_errors(tm, gemm):
+    K, N, T = 256, 64, 4
+    d = O.make_inputs(6600, T, K, N, 64)
+    qw, qz, s = dev(d["qweight"]), dev(d["qzeros"]), dev(d["scales"])
+    A, Q = torch.zeros_like(qw), torch.zeros_like(s, dtype=torch.int32)
+    tm.convert_s4_k_m8(A, Q, torch.zeros_like(s), qw, s, qz, N, K, 64)
+    C = torch.empty((T, N), dtype=torch.float16, device="cuda")
+    for bad in (256, 16, 96, 0):      # gemm_s4_f16.cu:119,233: the reference's message
+        with pytest.raises(tm.W4A16Error, match="unsupported group size") as e:
+            gemm.Run(C, A, dev(d["X"]), Q, N, T, K, bad)
+        assert e.value.code == -1
+    with pytest.raises(tm.W4A16Error, match="kernel ids belong to group size 128") as e:
+        gemm.Run(C, A, dev(d["X"]), Q, N, T, K, 64, 0, 0)
+    assert e.value.code == -5
+    with pytest.raises(tm.W4A16Error) as e:
+        gemm.Measure(C, A, dev(d["X"]), Q, N, T, K, 64)
+    assert e.value.code == -1
+
+
+def test_group_size_64_ffn_block(tm, gemm):
+    """w4a16_ffn (two GEMMs planned as a list) with group size 64, against the oracle."""
+    H, F, T, gs = 512, 1408, 9, 64
+    d13 = O.make_inputs(6700, T, H, 2 * F, gs, residual=True)
+    d2 = O.make_inputs(6701, T, F, H, gs)
+
+    def conv(dd, N, K):
+        qw, qz, s = dev(dd["qweight"]), dev(dd["qzeros"]), dev(dd["scales"])
+        A, Q = torch.zeros_like(qw), torch.zeros_like(s, dtype=torch.int32)
+        tm.convert_s4_k_m8(A, Q, torch.zeros_like(s), qw, s, qz, N, K, gs)
+        return A, Q
+    A13, Q13 = conv(d13, 2 * F, H)
+    A2, Q2 = conv(d2, H, F)
+    gating = torch.empty((T, F), dtype=torch.float16, device="cuda")
+    out = torch.empty((T, H), dtype=torch.float16, device="cuda")
+    res = dev(d13["R"][:, :H].copy())
+    gemm.ffn(out, gating, dev(d13["X"]), A13, Q13, A2, Q2, H, F, T, gs, residual=res)
+    torch.cuda.synchronize()
+    g_ref = O.gemm_s4_f16(d13["X"], d13["qweight"], d13["qzeros"], d13["scales"], gs, O.EPI_SILU)
+    assert_close(gating.cpu().numpy(), g_ref, "gating")
+    want = O.gemm_s4_f16(gating.cpu().numpy(), d2["qweight"], d2["qzeros"], d2["scales"], gs, O.EPI_ADD, d13["R"][:, :H])
+    assert_close(out.cpu().numpy(), want, "ffn output")

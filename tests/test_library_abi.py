@@ -50,7 +50,7 @@ def test_gemm_argument_validation(L):
     g = L.lib.w4a16_gemm
     assert g(None, P, P, P, P, None, 64, 4, 256, 128, 0, -1, None) == L.EARG and "null handle" in err(L)
     # gemm_s4_f16.cu:119,233: the reference's message for a group size it has no kernels for
-    assert g(FAKE, P, P, P, P, None, 64, 4, 256, 64, 0, -1, None) == L.EGROUP and err(L) == "unsupported group size"
+    assert g(FAKE, P, P, P, P, None, 64, 4, 256, 256, 0, -1, None) == L.EGROUP and err(L) == "unsupported group size"
     assert g(FAKE, P, P, P, P, None, 64, 4, 256, 128, 7, -1, None) == L.EARG
     assert g(FAKE, P, P, P, P, None, -1, 4, 256, 128, 0, -1, None) == L.EARG
     assert g(FAKE, None, P, P, P, None, 64, 4, 256, 128, 0, -1, None) == L.EARG
@@ -66,7 +66,7 @@ def test_gemm_argument_validation(L):
 
 def test_repack_argument_validation(L):
     lib = L.lib
-    assert lib.w4a16_convert_s4_k_m8(P, P, P, P, P, P, 64, 256, 32, None) == L.EGROUP
+    assert lib.w4a16_convert_s4_k_m8(P, P, P, P, P, P, 64, 256, 16, None) == L.EGROUP
     assert lib.w4a16_convert_s4_k_m8(P, P, P, P, P, P, 24, 256, 128, None) == L.ESHAPE
     assert lib.w4a16_convert_s4_k_m8(P, P, P, P, P, P, 64, 100, 128, None) == L.ESHAPE
     assert lib.w4a16_convert_s4_k_m8(None, P, P, P, P, P, 64, 256, 128, None) == L.EARG
@@ -77,14 +77,14 @@ def test_repack_argument_validation(L):
     assert lib.w4a16_transpose_qk_s4_k_m8_hf(P, P, 64, 4, 48, None) == L.ESHAPE      # 64 % 48 != 0
     assert lib.w4a16_dequantize_s4(None, P, 8, None) == L.EARG
     assert lib.w4a16_dequantize_s4(None, None, 0, None) == L.OK
-    assert lib.w4a16_unpack_repacked(P, P, P, P, P, 64, 256, 64, None) == L.EGROUP
+    assert lib.w4a16_unpack_repacked(P, P, P, P, P, 64, 256, 96, None) == L.EGROUP
     assert lib.w4a16_dequantize_repacked(None, P, P, 64, 256, 128, None) == L.EARG
     assert lib.w4a16_from_reference_layout(P, P, 48, 256, None) == L.ESHAPE          # m % 32
     assert lib.w4a16_reformat_s4_k_m8(P, None, 64, 256, None) == L.EARG
 
 
 def test_check_raises_with_code(L):
-    rc = L.lib.w4a16_gemm(FAKE, P, P, P, P, None, 64, 4, 256, 64, 0, -1, None)
+    rc = L.lib.w4a16_gemm(FAKE, P, P, P, P, None, 64, 4, 256, 512, 0, -1, None)
     with pytest.raises(L.W4A16Error, match="unsupported group size") as e:
         L.check(rc)
     assert e.value.code == L.EGROUP
@@ -115,7 +115,7 @@ def test_static_and_sequence_argument_validation(L):
     lib = L.lib
     # w4a16_gemm_static: the checks of w4a16_gemm, without a handle
     s = lib.w4a16_gemm_static
-    assert s(P, P, P, P, None, 64, 4, 256, 64, 0, -1, None) == L.EGROUP and err(L) == "unsupported group size"
+    assert s(P, P, P, P, None, 64, 4, 256, 256, 0, -1, None) == L.EGROUP and err(L) == "unsupported group size"
     assert s(P, P, P, P, None, 72, 4, 256, 128, 0, -1, None) == L.ESHAPE
     assert s(None, P, P, P, None, 64, 4, 256, 128, 0, -1, None) == L.EARG
     assert s(P, P, P, P, None, 64, 4, 256, 128, 2, -1, None) == L.EARG and "residual" in err(L)
@@ -129,7 +129,7 @@ def test_static_and_sequence_argument_validation(L):
     assert seq(None, one, 2, 4, 128, 0, None) == L.EARG and "null handle" in err(L)
     assert seq(FAKE, None, 2, 4, 128, 0, None) == L.EARG
     assert seq(FAKE, one, 2, 4, 128, 8, None) == L.EARG and "flags" in err(L)
-    assert seq(FAKE, one, 2, 4, 64, 0, None) == L.EGROUP
+    assert seq(FAKE, one, 2, 4, 48, 0, None) == L.EGROUP
     one[1].n_out = 72
     assert seq(FAKE, one, 2, 4, 128, L.SEQ_PERSISTENT, None) == L.ESHAPE
     one[1].n_out, one[1].epilogue = 64, 2
@@ -152,13 +152,13 @@ def test_deploy_entry_point_validation(L):
     lib = L.lib
     three = (ctypes.c_void_p * 3)(0x2000, 0x2000, 0x2000)
     q = lib.w4a16_deploy_qkv
-    assert q(P, P, three, three, three, 256, 256, 256, 128, 64, None) == L.EGROUP
+    assert q(P, P, three, three, three, 256, 256, 256, 128, 16, None) == L.EGROUP
     assert q(P, P, three, three, three, 256, 256, 256, 96, 128, None) == L.ESHAPE      # 256 % 96
     assert q(P, P, three, three, three, 256, 256, 200, 128, 128, None) == L.ESHAPE     # k % 128
     assert q(None, P, three, three, three, 256, 256, 256, 128, 128, None) == L.EARG
     assert q(P, P, (ctypes.c_void_p * 3)(0x2000, None, 0x2000), three, three, 256, 256, 256, 128, 128, None) == L.EARG
     assert q(None, None, None, None, None, 0, 0, 256, 128, 128, None) == L.OK          # empty
     w = lib.w4a16_deploy_w13
-    assert w(P, P, P, P, P, P, P, P, 64, 256, 32, None) == L.EGROUP
+    assert w(P, P, P, P, P, P, P, P, 64, 256, 256, None) == L.EGROUP
     assert w(P, P, P, P, P, P, P, P, 60, 256, 128, None) == L.ESHAPE                   # inter_size % 8
     assert w(P, P, P, None, P, P, P, P, 64, 256, 128, None) == L.EARG

@@ -128,7 +128,7 @@ def test_static_scratch_rejects_what_does_not_fit():
     want = O.gemm_s4_f16(d["X"], d["qweight"], d["qzeros"], d["scales"], 128)
     assert O.max_abs_rel(E.cpu().numpy(), want) <= TOL
     with pytest.raises(tm.W4A16Error) as e:
-        tm.gemm_static(C, A, X, Q, N, T, K, 64)
+        tm.gemm_static(C, A, X, Q, N, T, K, 256)
     assert e.value.code == -1
 
 
