@@ -437,28 +437,42 @@ struct GemmPlan {
     int     nq;  // quantisation groups per 128-row weight tile: 1 = the kernel table, 2 or 4 = the kernel for group size 64 / 32
 };
 
-// Group sizes 64 and 32 have one kernel (strips, gemm_strip.hip): nothing to choose, no scratch.
-int plan_small_groups(int n_out, int tokens, int k, int group_size, int algo_id, GemmPlan* out)
+// Group sizes 64 and 32 have two kernels outside the table (strips for few tokens, one MFMA tile for many): chosen
+// by rule, no scratch.
+constexpr int kGroupsStrips = -1, kGroupsMfma = -2;
+int plan_small_groups(const void* C, const void* R, int n_out, int tokens, int k, int group_size, int epilogue, int algo_id,
+                      GemmPlan* out)
 {
     if (algo_id >= 0)
         return fail(W4A16_EALGO, "kernel ids belong to group size 128; group size %d takes algo_id < 0 only", group_size);
     const int nq = 128 / group_size;
     if (!strip_groups_feasible(nq, n_out, tokens, k)) return fail(W4A16_ESHAPE, "no feasible kernel found");
-    out->algo = -1;
+    out->algo = kGroupsStrips;
     out->sc   = Scratch{};
     out->nq   = nq;
+    // Many tokens: the 256 x 128 MFMA tile (n_out a multiple of 128) once its K steps cost less than streaming the
+    // weights once per 16 tokens.  Step and stream figures measured on Llama-2-7B shapes with group size 64.
+    if (prefill_groups_feasible(nq, n_out, tokens, k)) {
+        const double tiles    = (double)((tokens + 255) / 256) * (n_out / 128);
+        const double mfma_us  = 3.0 + std::ceil(tiles / 256.0) * (k / 128) * 2.4;
+        const double strip_us = (double)((tokens + 15) / 16) * (3.0 + ((double)k * n_out / 2) / 3.0e6);
+        // (the MFMA kernel stores four features at a time: a pointer it cannot take leaves the GEMM with the strips)
+        const bool aligned = epilogue == W4A16_FUSED_SILU_FFN || (aligned8(C) && (!R || aligned8(R)));
+        if (mfma_us < strip_us && aligned) out->algo = kGroupsMfma;
+    }
     return W4A16_OK;
 }
 
 hipError_t launch_plan(const GemmPlan& plan, const GemmArgs& g, hipStream_t st)
 {
-    return plan.nq > 1 ? strip_groups_launch(plan.nq, g, st) : algo_launch(plan.algo, g, plan.sc, st);
+    if (plan.nq > 1) return plan.algo == kGroupsMfma ? prefill_groups_launch(plan.nq, g, st) : strip_groups_launch(plan.nq, g, st);
+    return algo_launch(plan.algo, g, plan.sc, st);
 }
 
 int plan_gemm(w4a16_handle* h, const void* C, const void* R, int n_out, int tokens, int k, int group_size, int epilogue,
               int algo_id, hipStream_t st, GemmPlan* out)
 {
-    if (group_size != 128) return plan_small_groups(n_out, tokens, k, group_size, algo_id, out);
+    if (group_size != 128) return plan_small_groups(C, R, n_out, tokens, k, group_size, epilogue, algo_id, out);
     out->nq = 1;
     if (algo_id >= algo_count()) return fail(W4A16_EALGO, "algo_id %d out of range (0..%d)", algo_id, algo_count() - 1);
     const bool chosen = algo_id >= 0;
@@ -512,7 +526,7 @@ int w4a16_gemm_static(void* C, const void* A, const void* X, const void* Q, cons
     if (algo_id >= algo_count()) return fail(W4A16_EALGO, "algo_id %d out of range (0..%d)", algo_id, algo_count() - 1);
     if (group_size != 128) {  // one kernel, no scratch at all
         GemmPlan plan{};
-        if (int rc = plan_small_groups(n_out, tokens, k, group_size, algo_id, &plan)) return rc;
+        if (int rc = plan_small_groups(C, R, n_out, tokens, k, group_size, epilogue, algo_id, &plan)) return rc;
         GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
                    n_out,        tokens,             k,                  epilogue};
         const hipError_t e = launch_plan(plan, g, (hipStream_t)stream);

@@ -117,7 +117,10 @@ __device__ __forceinline__ float hi_float(uint64_t v) { return __builtin_bit_cas
 // LDS, dequantised weights - are requested and prepared during the previous one.  A 64-token tile
 // has only 4 * NTW MFMAs per k32 chunk, too few to cover the LDS latency; two chunks per sub-step
 // double the cover at the price of a second set of fragment registers.
-template<int TTILES, int NTW, int WAVES, int D, int KS, int EPI>
+// NQ = quantisation groups per 128-row weight tile: 1 (group size 128), 2 (64) or 4 (32).  A K step is still one
+// weight tile; with NQ > 1 every k32 chunk (or pair of chunks) of the tile has its own scale and zero point, which
+// are taken from the tile's NQ Q words right before the chunk is dequantised instead of once per K step.
+template<int TTILES, int NTW, int WAVES, int D, int KS, int EPI, int NQ = 1>
 __global__ void __launch_bounds__(64 * WAVES)
     __attribute__((amdgpu_waves_per_eu(TTILES * NTW * KS >= 16 && WAVES == 4 && (TTILES * NTW >= 32 || KS == 2) ? 1 : 2,
                                        TTILES * NTW * KS >= 16 && WAVES == 4 && (TTILES * NTW >= 32 || KS == 2) ? 1 : 2)))
@@ -195,21 +198,26 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) acc[tt][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
+    static_assert(NQ == 1 || NQ == 2 || NQ == 4, "group sizes 128, 64 and 32");
+    constexpr int NQW = NTW * NQ;  // Q words per K step: tile nt's are qv[nt * NQ ..]
     u32x4_t  w[D][NTW];  // weights and (scale, zero) words of the D groups in flight; stage = group index mod D
-    uint32_t q[D][NTW];
+    uint32_t q[D][NQW];
 #pragma unroll
-    for (int d = 0; d < D; ++d)
+    for (int d = 0; d < D; ++d) {
 #pragma unroll
-        for (int nt = 0; nt < NTW; ++nt) {
-            w[d][nt] = u32x4_t{0, 0, 0, 0};
-            q[d][nt] = 0;
-        }
+        for (int nt = 0; nt < NTW; ++nt) w[d][nt] = u32x4_t{0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < NQW; ++i) q[d][i] = 0;
+    }
 
-    auto issue_w = [&](u32x4_t (&ws_)[NTW], uint32_t (&qv)[NTW], int g) {
+    auto issue_w = [&](u32x4_t (&ws_)[NTW], uint32_t (&qv)[NQW], int g) {
         const char* wbase = reinterpret_cast<const char*>(A) + (int64_t)g * NT * 1024;
-        const char* qbase = reinterpret_cast<const char*>(Q) + (int64_t)g * N * 4;
+        const char* qbase = reinterpret_cast<const char*>(Q) + (int64_t)g * NQ * N * 4;
         static_for<0, NTW>([&](auto nt) { gload128<nt * 1024>(ws_[nt], w_off, wbase); });
-        static_for<0, NTW>([&](auto nt) { gload32<nt * 64>(qv[nt], q_off, qbase); });
+        static_for<0, NQW>([&](auto i) {
+            constexpr int nt = decltype(i)::value / NQ, sub = decltype(i)::value % NQ;
+            gload32<nt * 64>(qv[decltype(i)::value], q_off, qbase + (int64_t)sub * N * 4);
+        });
     };
     // the activation tile of group g, straight into the LDS buffer `xo` (no registers, no ds_write)
     auto issue_x = [&](uint8_t* xo, int g) {
@@ -218,30 +226,30 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
         for (int i = 0; i < XB; ++i) gload_lds128(lds_addr(xo) + (wave * XB + i) * 1024, x_off[i], xbase);
     };
     // the same requests one at a time (m = 0 .. 2 NTW + TTILES - 1), to be dealt out between MFMAs
-    constexpr int kVmOps = 2 * NTW + XB;
-    auto vm_op = [&](auto M, u32x4_t (&ws_)[NTW], uint32_t (&qv)[NTW], uint8_t* xo, const char* wbase, const char* qbase,
+    constexpr int kVmOps = NTW + NQW + XB;
+    auto vm_op = [&](auto M, u32x4_t (&ws_)[NTW], uint32_t (&qv)[NQW], uint8_t* xo, const char* wbase, const char* qbase,
                      const char* xbase) {
         constexpr int m = decltype(M)::value;
         if constexpr (m < NTW) {
             gload128<m * 1024>(ws_[m], w_off, wbase);
         }
-        else if constexpr (m < 2 * NTW) {
-            gload32<(m - NTW) * 64>(qv[m - NTW], q_off, qbase);
+        else if constexpr (m < NTW + NQW) {
+            constexpr int nt = (m - NTW) / NQ, sub = (m - NTW) % NQ;
+            gload32<nt * 64>(qv[m - NTW], q_off, qbase + (int64_t)sub * N * 4);
         }
         else {
-            constexpr int i = m - 2 * NTW;
+            constexpr int i = m - NTW - NQW;
             gload_lds128(lds_addr(xo) + (wave * XB + i) * 1024, x_off[i], xbase);
         }
     };
     // wait until at most `Pending` younger stages' loads are in flight, then release the stage's registers
-    auto wait_stage = [&](auto Pending, u32x4_t (&ws_)[NTW], uint32_t (&qv)[NTW]) {
+    auto wait_stage = [&](auto Pending, u32x4_t (&ws_)[NTW], uint32_t (&qv)[NQW]) {
         constexpr int n = decltype(Pending)::value * kVmOps;
         static_assert(n <= 63, "vmcnt is a 6-bit counter");
 #pragma unroll
-        for (int nt = 0; nt < NTW; ++nt) {
-            wait_vm<n>(ws_[nt]);
-            wait_vm<n>(qv[nt]);
-        }
+        for (int nt = 0; nt < NTW; ++nt) wait_vm<n>(ws_[nt]);
+#pragma unroll
+        for (int i = 0; i < NQW; ++i) wait_vm<n>(qv[i]);
     };
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
@@ -253,8 +261,9 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     half8_t xf[2][KS][TTILES];
     half2_t z1024[2][NTW], z64[2][NTW], sc[2][NTW];
 
-    auto split = [&](auto P_, uint32_t (&qv)[NTW]) {
+    auto split = [&](auto P_, uint32_t (&qv)[NQW]) {
         constexpr int P = decltype(P_)::value;
+        if constexpr (NQ > 1) return;  // (taken chunk by chunk inside dequant_op)
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) {
             half_t s;
@@ -266,9 +275,15 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     // (op = NTW * k + nt) so that they can be dealt out between the MFMAs of a sub-step:
     // k = 0: w >> 8;  1..4: (w & mask) | magic;  5..8: - (offset + zero);  9..12: * scale.
     uint32_t dq[NTW][5];
-    auto dequant_op = [&](auto P, auto J, auto OP, u32x4_t (&ws_)[NTW]) {
-        constexpr int p = decltype(P)::value, j = decltype(J)::value;
+    auto dequant_op = [&](auto P, auto J, auto OP, u32x4_t (&ws_)[NTW], uint32_t (&qv)[NQW]) {
+        // (NQ > 1: the zero points and the scale of word j's quantisation group replace parity p's for this word)
+        constexpr int p = NQ > 1 ? 0 : decltype(P)::value, j = decltype(J)::value;
         constexpr int nt = decltype(OP)::value % NTW, k = decltype(OP)::value / NTW;
+        if constexpr (k == 0 && NQ > 1) {
+            half_t s;
+            split_q(qv[nt * NQ + j * NQ / 4], z1024[0][nt], z64[0][nt], s);
+            sc[0][nt] = half2_t{s, s};
+        }
         if constexpr (k == 0) dq[nt][4] = ws_[nt][j] >> 8;
         else if constexpr (k <= 4) {
             constexpr int i  = k - 1;
@@ -286,8 +301,8 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
             wf[(j / KS) & 1][j % KS][nt][2 * i + 1] = r[1];
         }
     };
-    auto dequant = [&](auto P, auto J, u32x4_t (&ws_)[NTW]) {
-        static_for<0, 13 * NTW>([&](auto op) { dequant_op(P, J, op, ws_); });
+    auto dequant = [&](auto P, auto J, u32x4_t (&ws_)[NTW], uint32_t (&qv)[NQW]) {
+        static_for<0, 13 * NTW>([&](auto op) { dequant_op(P, J, op, ws_, qv); });
     };
     auto read_x = [&](auto J_, const uint8_t* xb) {
         constexpr int  J    = decltype(J_)::value;
@@ -322,7 +337,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
     split(I0{}, q[0]);
     static_for<0, KS>([&](auto kc) {
         read_x(kc, xs);
-        dequant(I0{}, kc, w[0]);
+        dequant(I0{}, kc, w[0], q[0]);
     });
 
     // One K step (a quantisation group, four k32 chunks in kSub sub-steps) on stage S: weights w[S],
@@ -349,7 +364,7 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
                     wait_lgkm0(xf[par][kk][tt], xf[par][kk][tt + 1], xf[par][kk][tt + 2], xf[par][kk][tt + 3]);
             const int   g2 = min(g + D, gend - 1);  // (the last steps re-read the last group: no branch)
             const char* wbase = reinterpret_cast<const char*>(A) + (int64_t)g2 * NT * 1024;
-            const char* qbase = reinterpret_cast<const char*>(Q) + (int64_t)g2 * N * 4;
+            const char* qbase = reinterpret_cast<const char*>(Q) + (int64_t)g2 * NQ * N * 4;
             const char* xbase = reinterpret_cast<const char*>(X) + (int64_t)g2 * 256;
             if constexpr (last) {
                 // stages S + 2 .. S + D - 1 may still be in flight behind stage S + 1
@@ -372,8 +387,8 @@ prefill_kernel(uint16_t* __restrict__ C, const u32x4_t* __restrict__ A, const ui
                 static_for<i * kOps / kSlots, (i + 1) * kOps / kSlots>([&](auto op) {
                     constexpr int word = decltype(op)::value / (13 * NTW);
                     using OP           = std::integral_constant<int, decltype(op)::value % (13 * NTW)>;
-                    if constexpr (!last) dequant_op(P{}, std::integral_constant<int, (sub + 1) * KS + word>{}, OP{}, w[S]);
-                    else dequant_op(PN{}, std::integral_constant<int, word>{}, OP{}, w[SN]);
+                    if constexpr (!last) dequant_op(P{}, std::integral_constant<int, (sub + 1) * KS + word>{}, OP{}, w[S], q[S]);
+                    else dequant_op(PN{}, std::integral_constant<int, word>{}, OP{}, w[SN], q[SN]);
                 });
                 // the next sub-step's activation fragments, requested during the first three quarters
                 // of this one; in the last sub-step also the loads of group g + D
@@ -535,7 +550,7 @@ constexpr Variant kVariants[] = {
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
-template<int TTILES, int NTW, int WAVES, int D, int KS>
+template<int TTILES, int NTW, int WAVES, int D, int KS, int NQ = 1>
 hipError_t launch_v(int splits, const GemmArgs& a, const Scratch& sc, hipStream_t st)
 {
     constexpr int TT = 16 * TTILES, TN = 16 * NTW * WAVES;
@@ -546,7 +561,7 @@ hipError_t launch_v(int splits, const GemmArgs& a, const Scratch& sc, hipStream_
     const u32x4_t* A4 = reinterpret_cast<const u32x4_t*>(a.A);
 #define W4A16_LAUNCH(EPI)                                                                                              \
     do {                                                                                                               \
-        auto                         kfn = prefill_kernel<TTILES, NTW, WAVES, D, KS, EPI>;                             \
+        auto                         kfn = prefill_kernel<TTILES, NTW, WAVES, D, KS, EPI, NQ>;                         \
         static std::atomic<uint64_t> raised{0}; /* per instantiation, one bit per device */                            \
         const hipError_t             e = raise_lds_limit(reinterpret_cast<const void*>(kfn), (int)lds, raised);        \
         if (e != hipSuccess) return e;                                                                                 \
@@ -617,6 +632,20 @@ hipError_t prefill_launch(int v, int splits, const GemmArgs& a, const Scratch& s
         case 5: return launch_v<4, 1, 8, 4, 2>(splits, a, sc, st);
         default: return launch_v<4, 2, 8, 4, 1>(splits, a, sc, st);
     }
+}
+
+// Group sizes 64 and 32 (nq = 2, 4): the 256-token x 128-feature tile, the one variant with registers to spare for
+// the extra Q words of a K step.
+bool prefill_groups_feasible(int nq, int N, int T, int K)
+{
+    return (nq == 2 || nq == 4) && prefill_feasible(1, 1, N, T, K, 0, 0);
+}
+
+hipError_t prefill_groups_launch(int nq, const GemmArgs& a, hipStream_t st)
+{
+    if (!prefill_groups_feasible(nq, a.N, a.T, a.K)) return hipErrorInvalidValue;
+    const Scratch none{};
+    return nq == 2 ? launch_v<16, 2, 4, 2, 1, 2>(1, a, none, st) : launch_v<16, 2, 4, 2, 1, 4>(1, a, none, st);
 }
 
 // Predicted run time in microseconds, from the measured step times: launch and epilogue, the K

@@ -169,5 +169,8 @@ size_t     prefill_scratch_bytes(int variant, int splits, int N, int T, int K);
 int        prefill_grid(int variant, int splits, int N, int T, int K);
 hipError_t prefill_launch(int variant, int splits, const GemmArgs& a, const Scratch& sc, hipStream_t st);
 double     prefill_estimate_us(int variant, int splits, int N, int T, int K);  // model fitted to measurements
+// the 256 x 128 prefill tile for group sizes 64 and 32 (nq = 2, 4); needs n_out % 128 == 0
+bool       prefill_groups_feasible(int nq, int N, int T, int K);
+hipError_t prefill_groups_launch(int nq, const GemmArgs& a, hipStream_t st);
 
 }  // namespace w4a16

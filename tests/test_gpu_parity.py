@@ -743,6 +743,35 @@ def test_group_sizes_64_and_32_gemm(tm, gemm, gs, K, N):
                 assert torch.equal(Cs.view(torch.int16), C.view(torch.int16))
 
 
+@pytest.mark.parametrize("gs", [64, 32])
+def test_group_sizes_64_and_32_many_tokens(tm, gemm, gs):
+    """Above a few hundred tokens these group sizes run on the 256 x 128 MFMA tile (the reference's exact fp16
+    weight, scale and zero point changing inside the K step): token counts on both sides of a tile boundary, odd
+    numbers of K steps, every epilogue, every output against the oracle; a matrix whose width is not a multiple of
+    128 and a misaligned output stay with the strips."""
+    for K, N, Ts in ((640, 512, (300, 512, 700)), (1024, 2048, (1000,)), (256, 400, (600,))):
+        d = O.make_inputs(6800 + gs + N, max(Ts), K, N, gs, residual=True)
+        qw, qz, s = dev(d["qweight"]), dev(d["qzeros"]), dev(d["scales"])
+        A, Q = torch.zeros_like(qw), torch.zeros_like(s, dtype=torch.int32)
+        tm.convert_s4_k_m8(A, Q, torch.zeros_like(s), qw, s, qz, N, K, gs)
+        W = O.dequant_from_awq(d["qweight"], d["qzeros"], d["scales"], gs)
+        for T in Ts:
+            X, R = dev(d["X"][:T]), dev(d["R"][:T])
+            acc = O.gemm_acc(d["X"][:T], W)
+            for kind in (0, 1, 2):
+                want = O.epilogue(acc, kind, d["R"][:T] if kind == 2 else None)
+                C = torch.full((T, N // 2 if kind == 1 else N), float("nan"), dtype=torch.float16, device="cuda")
+                gemm.Run(C, A, X, Q, N, T, K, gs, kind, -1, residual=R if kind == 2 else None)
+                torch.cuda.synchronize()
+                assert_close(C.cpu().numpy(), want, (gs, K, N, T, kind))
+            if N % 128 == 0:
+                buf = torch.zeros(T * N + 8, dtype=torch.float16, device="cuda")
+                C1 = buf[2:2 + T * N].view(T, N)      # 4-byte aligned only
+                gemm.Run(C1, A, X, Q, N, T, K, gs, 0, -1)
+                torch.cuda.synchronize()
+                assert_close(C1.cpu().numpy(), O.epilogue(acc, 0), (gs, K, N, T, "misaligned"))
+
+
 def test_group_size_errors(tm, gemm):
     K, N, T = 256, 64, 4
     d = O.make_inputs(6600, T, K, N, 64)
