@@ -135,8 +135,23 @@ constexpr int kInPasses = 3;  // value of `per_cu` that asks for one workgroup p
 
 // `per_cu` strips per CU are aimed for; more if a strip would otherwise be wider than the limit.
 // block_t = tokens per workgroup: 16 (activation rows padded down to 4 or 8 for fewer tokens) or 32.
+// Compute units of the current device (the strips are dealt to that many workgroups, or a multiple): asked
+// once per device; 256, MI355X's count, where no device can be asked.
+int device_cus()
+{
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return kNumCU;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n > 0) return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = kNumCU;
+    cached[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
+
 StripPlan make_plan(int per_cu, int block_t, int N, int T, int K, int maxr_limit = kMaxR)
 {
+    const int cus = device_cus();
     StripPlan pl{};
     if (N <= 0 || K <= 0 || T <= 0 || N % kTileN != 0 || K % kGroup != 0 || per_cu < 1) return pl;
     if (block_t != 16 && block_t != 32) return pl;
@@ -144,22 +159,22 @@ StripPlan make_plan(int per_cu, int block_t, int N, int T, int K, int maxr_limit
     const int NT   = N / kTileN;
     const int maxr = std::min(maxr_limit, block_t == 32 ? kMaxR32 : kMaxR);
     int       m    = per_cu == kInPasses ? 1 : per_cu;
-    while ((NT + kNumCU * m - 1) / (kNumCU * m) > maxr) ++m;
-    pl.strips = std::min(NT, kNumCU * m);
+    while ((NT + cus * m - 1) / (cus * m) > maxr) ++m;
+    pl.strips = std::min(NT, cus * m);
     pl.base   = NT / pl.strips;
     pl.rem    = NT % pl.strips;
     pl.rmax   = pl.base + (pl.rem ? 1 : 0);
     pl.passes = 1;
     // 32-bit per-lane offsets into X; grid limits
     pl.ok = (int64_t)T * K * 2 < (1ll << 32) && (T + block_t - 1) / block_t <= 65535 &&
-            (per_cu == 1 || pl.strips == kNumCU * m);
+            (per_cu == 1 || pl.strips == cus * m);
     if (per_cu == kInPasses) {
         // Matrices too wide for one strip per CU: instead of m workgroups per CU side by side (16 or more waves
         // per CU asking for memory at once), one workgroup per CU takes its m strips in turn.  A plain streaming
         // read of 244 MiB is 10 % faster from 8 waves per CU than from 16.
         pl.ok     = pl.ok && m >= 2;
         pl.passes = m;
-        pl.strips = kNumCU;  // workgroups; base and rem still describe all m * 256 strips
+        pl.strips = cus;  // workgroups; base and rem still describe all m * cus strips
     }
     return pl;
 }

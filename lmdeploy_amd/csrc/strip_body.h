@@ -23,7 +23,7 @@ namespace strip {
 constexpr int kWaves   = 8;  // = K slices per workgroup
 constexpr int kMaxR    = 8;  // column tiles per strip
 constexpr int kMaxR32  = 8;  // ... with 32 tokens per workgroup
-constexpr int kNumCU   = 256;
+constexpr int kNumCU   = 256;  // MI355X; the deal itself asks the device (gemm_strip.hip)
 constexpr int kDmaTokens = 32;  // token block from which the activations go straight to LDS
 
 struct StripParams {
