@@ -41,7 +41,7 @@ MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16 matrix
 N_LAYERS = 32          # Llama-2-7B
 TRAFFIC_DECODE_GATE_UP = 49.36e6
 TRAFFIC_DECODE_O = 10.02e6
-TRAFFIC_PREFILL_GATE_UP = 567.7e6
+TRAFFIC_PREFILL_GATE_UP = 567.5e6
 
 # name, K, N (gate_up: both halves), epilogue
 LAYER_7B = [("qkv", 4096, 12288, 0), ("o", 4096, 4096, 0), ("gate_up", 4096, 22016, 1), ("down", 11008, 4096, 2)]

@@ -88,10 +88,40 @@ def main():
         for n in range(N):
             add[t, n] = float(R[t, n]) + float(Yh[t, n])
 
+    # The same weights and activations with a zero point and a scale per 32 rows (group size 32; drawn after
+    # everything above, so that the arrays above keep their values): Q words, dequantised weights and the plain
+    # GEMM, by the same element-wise rules.  The weight layout does not depend on the group size.
+    G32 = K // 32
+    z32 = rng.integers(0, 16, size=(G32, N))
+    s32 = (np.abs(rng.standard_normal((G32, N))) * 0.01 + 1e-3).astype(np.float16)
+    qzeros32 = np.zeros((G32, N // 8), dtype=np.uint32)
+    for g in range(G32):
+        for j in range(N // 8):
+            word = 0
+            for i in range(8):
+                word |= int(z32[g, 8 * j + ORDER[i]]) << (4 * i)
+            qzeros32[g, j] = word
+    Q32 = np.zeros((G32, N), dtype=np.uint32)
+    for g in range(G32):
+        for n in range(N):
+            Q32[g, n] = (0x5400 | (int(z32[g, n]) << 4)) | (int(s32[g, n:n + 1].view(np.uint16)[0]) << 16)
+    W32 = np.zeros((K, N), dtype=np.float16)
+    for k in range(K):
+        for n in range(N):
+            W32[k, n] = np.float16(np.float32(int(q[k, n]) - int(z32[k // 32, n])) * np.float32(s32[k // 32, n]))
+    Y32 = np.zeros((T, N), dtype=np.float64)
+    for t in range(T):
+        for n in range(N):
+            acc = 0.0
+            for k in range(K):
+                acc += float(X[t, k]) * float(W32[k, n])
+            Y32[t, n] = acc
+
     out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "w4a16_kat.npz")
     np.savez_compressed(out, K=K, N=N, T=T, q=q.astype(np.uint8), z=z.astype(np.uint8), scales=s, X=X, R=R,
                         qweight=qweight, qzeros=qzeros, Q=Q, W_bits=W.view(np.uint16), A_gfx950=A,
-                        Y=Y, Y_silu=silu, Y_add=add)
+                        Y=Y, Y_silu=silu, Y_add=add,
+                        z32=z32.astype(np.uint8), scales32=s32, qzeros32=qzeros32, Q32=Q32, W32_bits=W32.view(np.uint16), Y32=Y32)
     print("wrote", out, os.path.getsize(out), "bytes")
 
 

@@ -45,6 +45,18 @@ def test_oracle_gemm(kat, kind, key):
     assert got.shape == kat[key].shape and rel(got, kat[key]) <= 2e-3      # fp16 output against float64
 
 
+def test_oracle_group_size_32(kat):
+    from oracle import w4a16_oracle as O
+    K, N = int(kat["K"]), int(kat["N"])
+    assert np.array_equal(O.awq_pack(kat["z32"]), kat["qzeros32"])
+    W = O.dequant_from_awq(kat["qweight"], kat["qzeros32"], kat["scales32"], 32)
+    assert np.array_equal(W.view(np.uint16), kat["W32_bits"])
+    A, Q = O.convert_s4_k_m8(kat["qweight"], kat["scales32"], kat["qzeros32"], N, K, 32)
+    assert np.array_equal(A, kat["A_gfx950"]) and np.array_equal(Q, kat["Q32"])
+    got = O.gemm_s4_f16(kat["X"], kat["qweight"], kat["qzeros32"], kat["scales32"], 32)
+    assert rel(got, kat["Y32"]) <= 2e-3
+
+
 # ------------------------------------------------------------------ the library against the vectors (GPU)
 @pytest.fixture(scope="module")
 def gpu(kat):
@@ -90,3 +102,21 @@ def test_library_gemm_every_kernel(kat, gpu, kind, key):
         assert np.isfinite(got).all() and rel(got, kat[key]) <= TOL, (algo, rel(got, kat[key]))
         ran += 1
     assert ran >= 10
+
+
+@pytest.mark.gpu
+def test_library_group_size_32(kat, gpu):
+    torch, tm, dev = gpu["torch"], gpu["tm"], gpu["dev"]
+    K, N, T = gpu["K"], gpu["N"], int(kat["T"])
+    qw, qz, s = dev(kat["qweight"]), dev(kat["qzeros32"]), dev(kat["scales32"])
+    A, Q = torch.zeros_like(qw), torch.zeros_like(s, dtype=torch.int32)
+    tm.convert_s4_k_m8(A, Q, torch.zeros_like(s), qw, s, qz, N, K, 32)
+    assert np.array_equal(A.cpu().numpy().view(np.uint32).reshape(-1), kat["A_gfx950"])
+    assert np.array_equal(Q.cpu().numpy().view(np.uint32), kat["Q32"])
+    W = tm.dequantize_repacked(A, Q, N, K, 32).cpu().numpy()
+    assert np.array_equal(W.view(np.uint16), kat["W32_bits"])
+    C = torch.full((T, N), float("nan"), dtype=torch.float16, device="cuda")
+    tm.GemmS4F16().Run(C, A, dev(kat["X"]), Q, N, T, K, 32, 0, -1)
+    torch.cuda.synchronize()
+    got = C.cpu().numpy()
+    assert np.isfinite(got).all() and rel(got, kat["Y32"]) <= TOL
