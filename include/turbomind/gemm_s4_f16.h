@@ -153,6 +153,23 @@ public:
         }
     }
 
+    // Extensions (the reference's Measure only reports): what Measure found fastest on this object, kept in a
+    // text file across processes.  Both return the number of shapes written / taken over; LoadTuning throws
+    // std::runtime_error for a file measured with another library version or on another GPU model.
+    int SaveTuning(const std::string& path) const
+    {
+        const int rc = w4a16_save_tuning(h_, path.c_str());
+        raise(rc);
+        return rc;
+    }
+
+    int LoadTuning(const std::string& path)
+    {
+        const int rc = w4a16_load_tuning(h_, path.c_str());
+        raise(rc);
+        return rc;
+    }
+
 private:
     // gemm_s4_f16.cu:119,227,229,233: the same exception types and messages
     static void raise(int rc)

@@ -13,6 +13,7 @@
 #include <cstring>
 #include <sstream>
 #include <type_traits>
+#include <string>
 #include <vector>
 
 namespace turbomind {
@@ -143,6 +144,13 @@ int main()
                 std::printf("Measure returned %zu rows, fastest id %d: %s\n", metrics.size(), metrics.empty() ? -1 : metrics[0].id,
                             ok ? "ok" : "FAILED");
                 failed += !ok;
+                // what Measure learnt survives in a file: a second object loads it and makes the same choice
+                const std::string path = "/tmp/w4a16_dropin_tuning.txt";
+                const int         saved = gemm.SaveTuning(path);
+                GemmS4F16         other;
+                const int         loaded = other.LoadTuning(path);
+                std::printf("tuning file: saved %d, loaded %d: %s\n", saved, loaded, saved == 1 && loaded == 1 ? "ok" : "FAILED");
+                failed += !(saved == 1 && loaded == 1);
             }
             (void)hipFree(X);
             (void)hipFree(R);

@@ -41,4 +41,5 @@ def test_llama_linear_shaped_caller_computes_the_known_answers():
         assert ("drop-in GEMM ran, tokens %d: kGemm mismatches 0, kFusedSiluFfn mismatches 0 (+0 written past the output), "
                 "kFusedAdd mismatches 0" % T) in r.stdout
     assert 'group size 256: "unsupported group size" ok' in r.stdout
+    assert "tuning file: saved 1, loaded 1: ok" in r.stdout
     assert "drop-in checks passed" in r.stdout
