@@ -238,6 +238,12 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     constexpr int kLoads = R + R * NQ + NX;  // loads per stage
 
     const UnpackConsts uc;
+    // B operand of the chain that sums the activations: -(unpack offset) in columns 0-7, -1 in columns 8-15
+    half8_t bsum;
+    {
+        const half_t lo = c < 8 ? (half_t)-1024.f : (half_t)-1.f, hi = c < 8 ? (half_t)-64.f : (half_t)-1.f;
+        bsum = half8_t{lo, lo, hi, hi, lo, lo, hi, hi};
+    }
     float4_t           acc[H][R];
 #pragma unroll
     for (int h = 0; h < H; ++h)
@@ -273,41 +279,78 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
 #pragma unroll
                 for (int j = 0; j < 4; ++j) xf[h][j] = __builtin_bit_cast(half8_t, xw[xr_at[h][j]]);  // same wave: LDS keeps the order
         }
-        constexpr int U = 2;
+        constexpr int U  = 2;
+        constexpr int JN = 4 / NQ;  // k32 chunks per quantisation group
+        // What the unpack offsets and the zero points add to every dot product depends on the weights only
+        // through z: sum x (q + o) - P - z S = sum x (q - z) with P = sum o x (o = 1024 under the low-nibble
+        // pairs, 64 under the high ones) and S = sum x.  A strip of two or more tiles takes P and S from one
+        // MFMA chain per quantisation group (columns 0-7 of its B operand hold -o, columns 8-15 hold -1) and
+        // every tile starts its own chain from -P: four MFMAs per tile instead of eight.  A strip of one tile
+        // runs the second chain per tile, with -(o + z) as its B operand; that costs it no more MFMAs and
+        // saves the exchange between the two halves of the columns.
+        constexpr bool kSums = R >= 2;
 #pragma unroll
-        for (int r0 = 0; r0 < R; r0 += U) {
+        for (int sub = 0; sub < NQ; ++sub) {  // the rows of the tiles that share a scale and a zero point
+            float4_t nP[H], nS[H];
+            if constexpr (kSums) {
 #pragma unroll
-            for (int sub = 0; sub < NQ; ++sub) {  // the rows of the tile that share a scale and a zero point
-                constexpr int JN = 4 / NQ;        // k32 chunks per quantisation group
+                for (int h = 0; h < H; ++h) {
+                    float4_t ps = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int j = sub * JN; j < (sub + 1) * JN; ++j)
+                        ps = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[h][j], bsum, ps, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        // the lane eight columns away, row_ror:8 (source given as the old value too: with a constant
+                        // there the compiler merges the four moves into one)
+                        const int   mine  = __builtin_bit_cast(int, (float)ps[i]);
+                        const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(mine, mine, 0x128, 0xf, 0xf, false));
+                        nP[h][i] = c < 8 ? ps[i] : other;
+                        nS[h][i] = c < 8 ? other : ps[i];
+                    }
+                }
+            }
+#pragma unroll
+            for (int r0 = 0; r0 < R; r0 += U) {
                 float4_t g4[H][U];
-                float    sf[U];
+                float    sf[U], zf[U];
                 half8_t  bz[U];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const int      r  = r0 + u < R ? r0 + u : R - 1;
-                    const uint32_t qw = s.q[r * NQ + sub];
-                    // B operand that removes the unpack offsets and the zero point: -(1024 + z) under
-                    // the low-nibble pairs, -(64 + z) under the high-nibble pairs
-                    const half2_t  h2  = as_half2(qw);
-                    const half2_t  n64 = half2_t{h2[0], h2[0]} * half2_t{(half_t)-1.f, (half_t)-1.f};
-                    const uint32_t zb  = ((qw >> 4) & 0xfu) * 0x10001u + 0xE400E400u;  // -(1024 + z) twice
-                    bz[u][0] = as_half2(zb)[0]; bz[u][1] = as_half2(zb)[1]; bz[u][2] = n64[0]; bz[u][3] = n64[1];
-                    bz[u][4] = bz[u][0]; bz[u][5] = bz[u][1]; bz[u][6] = bz[u][2]; bz[u][7] = bz[u][3];
+                    const uint32_t qw = s.q[r * NQ + sub];  // half2(64 + z, scale): z is bits 4-7
+                    const half2_t  h2 = as_half2(qw);
+                    if constexpr (kSums) {
+                        zf[u] = (float)((qw >> 4) & 0xfu);
+                        asm volatile("" : "+v"(zf[u]));
+                    }
+                    else {
+                        // -(1024 + z) under the low-nibble pairs, -(64 + z) under the high-nibble pairs
+                        const half2_t  n64 = half2_t{h2[0], h2[0]} * half2_t{(half_t)-1.f, (half_t)-1.f};
+                        const uint32_t zb  = ((qw >> 4) & 0xfu) * 0x10001u + 0xE400E400u;  // -(1024 + z) twice
+                        bz[u][0] = as_half2(zb)[0]; bz[u][1] = as_half2(zb)[1]; bz[u][2] = n64[0]; bz[u][3] = n64[1];
+                        bz[u][4] = bz[u][0]; bz[u][5] = bz[u][1]; bz[u][6] = bz[u][2]; bz[u][7] = bz[u][3];
+                    }
                     // Convert the scale now and hide it from the optimiser: otherwise the conversion is
                     // folded into the final multiply-add, the Q word stays live past the refill of this
                     // stage, and the refill lands in a copy that is moved back while still in flight.
                     sf[u] = scale_is_normal(qw) ? (float)h2[1] : 0.f;
                     asm volatile("" : "+v"(sf[u]));
 #pragma unroll
-                    for (int h = 0; h < H; ++h) g4[h][u] = float4_t{0.f, 0.f, 0.f, 0.f};
+                    for (int h = 0; h < H; ++h) {
+                        if constexpr (kSums) g4[h][u] = nP[h];
+                        else g4[h][u] = float4_t{0.f, 0.f, 0.f, 0.f};
+                    }
                 }
+                if constexpr (!kSums) {
 #pragma unroll
-                for (int j = sub * JN; j < (sub + 1) * JN; ++j) {
+                    for (int j = sub * JN; j < (sub + 1) * JN; ++j) {
 #pragma unroll
-                    for (int u = 0; u < U; ++u)
+                        for (int u = 0; u < U; ++u)
 #pragma unroll
-                        for (int h = 0; h < H; ++h)
-                            if (r0 + u < R) g4[h][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[h][j], bz[u], g4[h][u], 0, 0, 0);
+                            for (int h = 0; h < H; ++h)
+                                if (r0 + u < R) g4[h][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[h][j], bz[u], g4[h][u], 0, 0, 0);
+                    }
                 }
 #pragma unroll
                 for (int j = sub * JN; j < (sub + 1) * JN; ++j) {
@@ -329,7 +372,10 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
                 for (int u = 0; u < U; ++u)
 #pragma unroll
                     for (int h = 0; h < H; ++h)
-                        if (r0 + u < R) acc[h][r0 + u] += sf[u] * g4[h][u];
+                        if (r0 + u < R) {
+                            if constexpr (kSums) acc[h][r0 + u] += sf[u] * (g4[h][u] + zf[u] * nS[h]);
+                            else acc[h][r0 + u] += sf[u] * g4[h][u];
+                        }
             }
         }
     };
