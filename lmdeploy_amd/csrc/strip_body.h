@@ -251,7 +251,7 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
         for (int r = 0; r < R; ++r) acc[h][r] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     // One tile of one group.  U tiles are worked on at a time with their MFMA chains interleaved:
-    // a chain is eight dependent MFMAs, and a dependent MFMA cannot issue before its predecessor
+    // a chain is four or eight dependent MFMAs, and a dependent MFMA cannot issue before its predecessor
     // has left the pipe.
     auto compute = [&](StageT& s, auto dc) {
         half8_t xf[H][4];
