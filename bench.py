@@ -210,6 +210,15 @@ def main():
         ms = sorted(timed_all(runner, steps, warmup, repeats))
         return ms[len(ms) // 2]
 
+    def kernel_clock(work, fn=None, steps=3):
+        """The engine clock inside the kernels of `work` (a launch list as for make_runner): the graph is captured and
+        replayed with the library's clock recording on, apart from the timed regions."""
+        gemm.clock_begin(stream.cuda_stream)
+        r = make_runner([work], fn)
+        timed(r, steps, 1, 1)
+        c = gemm.clock_end(stream.cuda_stream)
+        return {"MHz": round(c["MHz"]), "kernel_us": round(c["us_per_launch"], 2)} if c["launches"] else None
+
     if args.probe and args.probe.startswith("sustain-"):
         K, N, _ = shape["gate_up"]
         T = 8 if args.probe == "sustain-decode" else PREFILL_T
@@ -481,13 +490,38 @@ def main():
                 torch.cuda.synchronize()
                 barrier[kind + "_us"] = round(e0.elapsed_time(e1) * 1e3 / 2000, 3)
         gemm.sequence_status(stream.cuda_stream)
+        # the matrix pipes alone (w4a16_probe_mfma: nothing but MFMAs on registers) and the clock they run at
+        mfma_loop = {}
+        with torch.cuda.stream(stream):
+            for waves in (8, 16):
+                gemm.probe_mfma(waves, 2000)
+                gemm.clock_begin(stream.cuda_stream)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                torch.cuda.synchronize()
+                e0.record(stream)
+                fl = sum(gemm.probe_mfma(waves, 40000) for _ in range(8))
+                e1.record(stream)
+                c = gemm.clock_end(stream.cuda_stream)
+                tf = fl / e0.elapsed_time(e1) / 1e9
+                mfma_loop["waves_per_cu_%d" % waves] = {"TFLOPs": round(tf, 1), "frac": round(tf / MFMA_PEAK_TFLOPS, 3),
+                                                        "engine_clock_MHz": round(c["MHz"])}
+        # the engine clock inside a streaming read and inside the decode kernel of gate_up
+        bufs = [torch.zeros(45 << 20, dtype=torch.uint8, device="cuda") for _ in range(max(3, int(args.cold_gib * 1024 / 45) + 1))]
+        clocks = {"read_45MiB_wg1_inflight4_nt": kernel_clock(bufs, lambda w, st: [gemm.probe_stream(b, 1, 4, 1, stream=st) for b in w])}
+        del bufs
+        for T in (1, 16):
+            clocks["gate_up_T%d" % T] = kernel_clock([("gate_up", c, T) for c in range(len(weights["gate_up"]))])
         ceilings = dict(reads, device_wide_barrier=barrier, device_copy_512MiB_GBps=round(copy_gbs, 1),
+                        mfma_loop=mfma_loop, engine_clock_in_kernel=clocks,
                         dense_fp16_gemm_gate_up_T2048_TFLOPs=round(dense_tf, 1),
                         note="read_*: w4a16_probe_read (plain streaming read, one launch per buffer in a HIP graph, cold buffers) and, "
                              "under counted_loads_us, w4a16_probe_stream (the GEMM kernels' load pipeline: wgN = workgroups of eight "
                              "waves per CU, inflightN = 16-byte loads per lane kept in flight, nt = non-temporal); "
                              "device_wide_barrier: w4a16_probe_barrier, one workgroup per CU, 2000 barriers in one launch; "
-                             "torch copy_ (bytes read + written); torch.matmul fp16 (hipBLASLt)")
+                             "torch copy_ (bytes read + written); torch.matmul fp16 (hipBLASLt); mfma_loop: w4a16_probe_mfma, "
+                             "8 launches of 40000 x 4 MFMAs per wave; engine_clock_in_kernel (and llama70b rows): core-clock "
+                             "cycles over constant-rate ticks between the first and last instruction of one wave per launch "
+                             "(w4a16_probe_clock_begin / _end), kernel_us = those ticks per launch")
 
     # ---- Llama-2-70B layer shapes (BASELINE configs[3]) -----------------------------------------
     llama70b = None
@@ -511,7 +545,8 @@ def main():
                 us = timed(make_runner([[(c, T) for c in range(n)]], run70), 3, 1, 5) * 1e3 / (3 * n)
                 by = algorithmic_bytes(T, K, N, epi)
                 rows70.append({"shape": name, "T": T, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
-                               "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 3)})
+                               "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 3),
+                               "engine_clock": kernel_clock([(c, T) for c in range(n)], run70)})
             us = timed(make_runner([[(c, PREFILL_T) for c in range(n)]], run70), 2, 1, 3) * 1e3 / (2 * n)
             fl = flops(PREFILL_T, K, N)
             rows70.append({"shape": name, "T": PREFILL_T, "us": round(us, 1), "TFLOPs": round(fl / us / 1e6, 1),

@@ -4,7 +4,8 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_size_t, c_void_p
+from ctypes import (POINTER, Structure, c_char_p, c_double, c_float, c_int, c_longlong, c_size_t, c_ulonglong,
+                    c_void_p)
 
 # The callers hand over torch tensors, so torch is in the process anyway - and it must come first:
 # torch ships its own libamdhip64 and libw4a16.so has to bind to that same HIP runtime.  Loaded the
@@ -69,6 +70,10 @@ SIGNATURES = {
     "w4a16_probe_read": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "w4a16_probe_stream": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_void_p]),
     "w4a16_probe_barrier": (c_int, [c_void_p, c_int, c_int, c_void_p]),
+    "w4a16_probe_mfma": (c_int, [c_void_p, c_int, c_int, c_void_p]),
+    "w4a16_probe_clock_begin": (c_int, [c_void_p, c_void_p]),
+    "w4a16_probe_clock_end": (c_int, [c_void_p, POINTER(c_ulonglong), POINTER(c_ulonglong), POINTER(c_ulonglong),
+                                      POINTER(c_longlong), c_void_p]),
     "w4a16_last_error": (c_char_p, []),
     "w4a16_version": (c_char_p, []),
 }

@@ -60,6 +60,8 @@ struct w4a16_handle {
     int            cus{};         // compute units of the device: workgroups of a persistent launch
     long long      clock_khz{};   // rate of the device's wall clock
     long long      spin_ticks{};  // time limit of one barrier wait
+    unsigned long long* clk{};    // measurement aid: cycle, tick and launch counters of w4a16_probe_clock_*
+    bool           clk_on{};      // strip kernels and probes launched through this handle record into them
     // fastest kernel found by w4a16_measure, per (n_out, tokens, k); consulted before the heuristic
     std::map<std::tuple<int, int, int>, int> tuned;
 };
@@ -329,6 +331,8 @@ int w4a16_create(w4a16_handle** out)
     if (e == hipSuccess) e = hipMemset(h->scratch.cnt, 0, kCounters * sizeof(int));
     if (e == hipSuccess) e = hipMalloc((void**)&h->sync, kSyncInts * sizeof(int));
     if (e == hipSuccess) e = hipMemset(h->sync, 0, kSyncInts * sizeof(int));
+    if (e == hipSuccess) e = hipMalloc((void**)&h->clk, 4 * sizeof(unsigned long long));
+    if (e == hipSuccess) e = hipMemset(h->clk, 0, 4 * sizeof(unsigned long long));
     if (e == hipSuccess) e = hipDeviceGetAttribute(&h->cus, hipDeviceAttributeMultiprocessorCount, h->device);
     int khz = 0;
     if (e == hipSuccess) e = hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, h->device);
@@ -343,6 +347,7 @@ int w4a16_create(w4a16_handle** out)
         if (h->ev_end) (void)hipEventDestroy(h->ev_end);
         if (h->scratch.cnt) (void)hipFree(h->scratch.cnt);
         if (h->sync) (void)hipFree(h->sync);
+        if (h->clk) (void)hipFree(h->clk);
         delete h;
         return hip_fail(e, "w4a16_create");
     }
@@ -361,6 +366,7 @@ void w4a16_destroy(w4a16_handle* h)
     if (h->scratch.ws) (void)hipFree(h->scratch.ws);
     (void)hipFree(h->scratch.cnt);
     (void)hipFree(h->sync);
+    (void)hipFree(h->clk);
     delete h;
 }
 
@@ -512,6 +518,7 @@ int w4a16_gemm(w4a16_handle* h, void* C, const void* A, const void* X, const voi
     if (int rc = plan_gemm(h, C, R, n_out, tokens, k, group_size, epilogue, algo_id, (hipStream_t)stream, &plan)) return rc;
     GemmArgs g{(uint16_t*)C, (const uint32_t*)A, (const uint16_t*)X, (const uint32_t*)Q, (const uint16_t*)R,
                n_out,        tokens,             k,                  epilogue};
+    if (h->clk_on) g.clk = h->clk;
     const hipError_t e = launch_plan(plan, g, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "w4a16_gemm launch");
     return W4A16_OK;
@@ -853,8 +860,45 @@ int w4a16_probe_stream(w4a16_handle* h, const void* src, size_t bytes, int wg_pe
         return fail(W4A16_EARG, "probe_stream: wg_per_cu is 1, 2 or 4, in_flight 2, 4, 8 or 16, hint 0, 1 or 2");
     if (h->cus > 256) return fail(W4A16_ESHAPE, "probe_stream: more than 256 CUs");
     if (int rc = check_device(h)) return rc;
-    const hipError_t e = launch_probe_stream(src, bytes, h->sync + 64 * 40, h->cus, wg_per_cu, in_flight, hint, (hipStream_t)stream);
+    const hipError_t e = launch_probe_stream(src, bytes, h->sync + 64 * 40, h->cus, wg_per_cu, in_flight, hint, (hipStream_t)stream,
+                                             h->clk_on ? h->clk : nullptr);
     return e == hipSuccess ? W4A16_OK : hip_fail(e, "probe_stream");
+}
+
+int w4a16_probe_mfma(w4a16_handle* h, int waves_per_cu, int iters, void* stream)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    if (waves_per_cu != 4 && waves_per_cu != 8 && waves_per_cu != 16) return fail(W4A16_EARG, "probe_mfma: waves_per_cu is 4, 8 or 16");
+    if (iters < 1 || iters > (1 << 24)) return fail(W4A16_EARG, "probe_mfma: iters out of range");
+    if (int rc = check_device(h)) return rc;
+    const hipError_t e = launch_probe_mfma(h->sync + 64 * 40, h->cus, waves_per_cu, iters, h->clk_on ? h->clk : nullptr, (hipStream_t)stream);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e, "probe_mfma");
+}
+
+int w4a16_probe_clock_begin(w4a16_handle* h, void* stream)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    if (int rc = check_device(h)) return rc;
+    const hipError_t e = hipMemsetAsync(h->clk, 0, 4 * sizeof(unsigned long long), (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "probe_clock_begin");
+    h->clk_on = true;
+    return W4A16_OK;
+}
+
+int w4a16_probe_clock_end(w4a16_handle* h, unsigned long long* cycles, unsigned long long* ticks, unsigned long long* launches,
+                          long long* ticks_per_second, void* stream)
+{
+    if (!h) return fail(W4A16_EARG, "null handle");
+    if (!cycles || !ticks || !launches) return fail(W4A16_EARG, "probe_clock_end: null output pointer");
+    if (int rc = check_device(h)) return rc;
+    h->clk_on = false;
+    unsigned long long v[4] = {0, 0, 0, 0};
+    hipError_t e = hipStreamSynchronize((hipStream_t)stream);
+    if (e == hipSuccess) e = hipMemcpy(v, h->clk, sizeof(v), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return hip_fail(e, "probe_clock_end");
+    *cycles = v[0], *ticks = v[1], *launches = v[2];
+    if (ticks_per_second) *ticks_per_second = h->clock_khz * 1000;
+    return W4A16_OK;
 }
 
 int w4a16_probe_barrier(w4a16_handle* h, int iters, int tree, void* stream)

@@ -39,6 +39,7 @@ template<int RMAX, int TP, int EPI>
 __global__ void __launch_bounds__(64 * kWaves) strip_kernel(const StripParams p)
 {
     extern __shared__ __attribute__((aligned(16))) u32x4_t smem[];  // activation patches [8][1 or 2][TP][16], then sums [8][R][H][64]
+    clock_record_start(p.clk, blockIdx.x == gridDim.x / 2 && blockIdx.y == 0 && threadIdx.x == 0);
     for (int pass = 0; pass < p.passes; ++pass) {
         const int  bx   = pass * gridDim.x + blockIdx.x;
         const bool wide = bx < p.rem;
@@ -53,6 +54,7 @@ __global__ void __launch_bounds__(64 * kWaves) strip_kernel(const StripParams p)
         }
         if (!done) strip_body<RMAX, TP, EPI>(p, col0, smem);
     }
+    clock_record_stop(p.clk, blockIdx.x == gridDim.x / 2 && blockIdx.y == 0 && threadIdx.x == 0);
 }
 
 // The same kernel for group sizes 64 and 32 (NQ = 2, 4 quantisation groups per 128-row tile): 16 token rows per
@@ -204,7 +206,7 @@ hipError_t strip_launch(int per_cu, int block_t, const GemmArgs& a, hipStream_t 
     const int   tp = block_t == 32 ? 32 : (a.T <= 4 ? 4 : (a.T <= 8 ? 8 : 16));
     const int   h  = tp > 16 ? tp / 16 : 1;
     StripParams p{a.C, reinterpret_cast<const u32x4_t*>(a.A), a.X, a.Q, a.R, a.N, a.T, a.K, pl.base, pl.rem,
-                  a.epilogue, pl.passes};
+                  a.epilogue, pl.passes, a.clk};
     const dim3   grid(pl.strips, (a.T + block_t - 1) / block_t);
     // per wave: the sums of its strip, over its activation patch(es) - two for 32 tokens, which arrive straight from memory
     const size_t lds = (size_t)kWaves * std::max(pl.rmax * h * 1024, tp * 256 * (tp >= kDmaTokens ? 2 : 1));

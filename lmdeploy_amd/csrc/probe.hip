@@ -8,6 +8,8 @@
 // waited for by count, so that a constant number of them stays in flight per lane from the first
 // instruction to the last - with the number in flight, the workgroups per CU and the cache hint as
 // parameters, for sweeping what the memory system gives at best.
+// probe_mfma_kernel: nothing but v_mfma_f32_16x16x32_f16 on registers, for the rate the matrix pipes reach at
+// the clock the chip settles at under them.
 #include "w4a16_common.h"
 
 #include <algorithm>
@@ -64,8 +66,10 @@ __device__ __forceinline__ void probe_load(u32x4_t& dst, uint32_t voff, const vo
 // Every wave keeps U loads of 1 KiB in flight; block number i of wave w is w + i * (waves of the
 // grid), so at any moment the chip reads one contiguous window of the buffer.
 template<int U, int HINT>
-__global__ void __launch_bounds__(512) probe_stream_kernel(const char* __restrict__ src, int blocks, uint32_t* sink)
+__global__ void __launch_bounds__(512) probe_stream_kernel(const char* __restrict__ src, int blocks, uint32_t* sink,
+                                                           unsigned long long* clk)
 {
+    clock_record_start(clk, blockIdx.x == gridDim.x / 2 && threadIdx.x == 0);
     const int lane   = threadIdx.x & 63;
     const int wid    = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 8 + (threadIdx.x >> 6)));
     const int nwaves = gridDim.x * 8;
@@ -89,18 +93,49 @@ __global__ void __launch_bounds__(512) probe_stream_kernel(const char* __restric
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const uint32_t x = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
     if (x == 0x9e3779b9u) sink[blockIdx.x & 2047] = x;  // (keeps the loads alive; practically never taken)
+    clock_record_stop(clk, blockIdx.x == gridDim.x / 2 && threadIdx.x == 0);
 }
 
 template<int U>
-hipError_t launch_stream(int hint, const void* src, int blocks, void* sink, int grid, hipStream_t st)
+hipError_t launch_stream(int hint, const void* src, int blocks, void* sink, int grid, hipStream_t st, unsigned long long* clk)
 {
     const char* s = (const char*)src;
     uint32_t*   k = (uint32_t*)sink;
     switch (hint) {
-        case 0: return launch_kernel(probe_stream_kernel<U, 0>, dim3(grid), dim3(512), 0, st, s, blocks, k);
-        case 1: return launch_kernel(probe_stream_kernel<U, 1>, dim3(grid), dim3(512), 0, st, s, blocks, k);
-        default: return launch_kernel(probe_stream_kernel<U, 2>, dim3(grid), dim3(512), 0, st, s, blocks, k);
+        case 0: return launch_kernel(probe_stream_kernel<U, 0>, dim3(grid), dim3(512), 0, st, s, blocks, k, clk);
+        case 1: return launch_kernel(probe_stream_kernel<U, 1>, dim3(grid), dim3(512), 0, st, s, blocks, k, clk);
+        default: return launch_kernel(probe_stream_kernel<U, 2>, dim3(grid), dim3(512), 0, st, s, blocks, k, clk);
     }
+}
+
+// Four independent accumulator chains per wave, operands that change from one MFMA to the next (two fixed
+// pseudo-random fragment pairs in turn), `iters` rounds of four MFMAs.
+template<int WAVES>
+__global__ void __launch_bounds__(64 * WAVES) probe_mfma_kernel(float* sink, int iters, unsigned long long* clk)
+{
+    clock_record_start(clk, blockIdx.x == gridDim.x / 2 && threadIdx.x == 0);
+    half8_t a[2], b[2];
+    uint32_t seed = 0x9e3779b9u * (threadIdx.x + 1) + blockIdx.x;
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            seed     = seed * 1664525u + 1013904223u;
+            a[s][e]  = (half_t)((float)((seed >> 9) & 0xff) * (1.f / 256.f) - 0.5f);
+            seed     = seed * 1664525u + 1013904223u;
+            b[s][e]  = (half_t)((float)((seed >> 9) & 0xff) * (1.f / 256.f) - 0.5f);
+        }
+    float4_t acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < iters; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j & 1], b[(j >> 1) & 1], acc[j], 0, 0, 0);
+    }
+    const float4_t t = acc[0] + acc[1] + acc[2] + acc[3];
+    const float    x = t[0] + t[1] + t[2] + t[3];
+    if (x == 12345.678f) sink[blockIdx.x & 2047] = x;  // (keeps the chains alive; practically never taken)
+    clock_record_stop(clk, blockIdx.x == gridDim.x / 2 && threadIdx.x == 0);
 }
 
 }  // namespace
@@ -120,18 +155,30 @@ bool probe_stream_config_ok(int wg_per_cu, int in_flight, int hint)
            hint >= 0 && hint <= 2;
 }
 
+hipError_t launch_probe_mfma(void* sink, int cus, int waves_per_cu, int iters, unsigned long long* clk, hipStream_t st)
+{
+    if (iters < 1 || cus < 1) return hipErrorInvalidValue;
+    float* k = (float*)sink;
+    switch (waves_per_cu) {
+        case 4: return launch_kernel(probe_mfma_kernel<4>, dim3(cus), dim3(256), 0, st, k, iters, clk);
+        case 8: return launch_kernel(probe_mfma_kernel<8>, dim3(cus), dim3(512), 0, st, k, iters, clk);
+        case 16: return launch_kernel(probe_mfma_kernel<16>, dim3(cus), dim3(1024), 0, st, k, iters, clk);
+        default: return hipErrorInvalidValue;
+    }
+}
+
 hipError_t launch_probe_stream(const void* src, size_t bytes, void* sink, int cus, int wg_per_cu, int in_flight, int hint,
-                               hipStream_t st)
+                               hipStream_t st, unsigned long long* clk)
 {
     if (!probe_stream_config_ok(wg_per_cu, in_flight, hint) || bytes / 1024 > (size_t)INT32_MAX) return hipErrorInvalidValue;
     const int blocks = (int)(bytes / 1024);
     if (blocks == 0) return hipSuccess;
     const int grid = cus * wg_per_cu;
     switch (in_flight) {
-        case 2: return launch_stream<2>(hint, src, blocks, sink, grid, st);
-        case 4: return launch_stream<4>(hint, src, blocks, sink, grid, st);
-        case 8: return launch_stream<8>(hint, src, blocks, sink, grid, st);
-        default: return launch_stream<16>(hint, src, blocks, sink, grid, st);
+        case 2: return launch_stream<2>(hint, src, blocks, sink, grid, st, clk);
+        case 4: return launch_stream<4>(hint, src, blocks, sink, grid, st, clk);
+        case 8: return launch_stream<8>(hint, src, blocks, sink, grid, st, clk);
+        default: return launch_stream<16>(hint, src, blocks, sink, grid, st, clk);
     }
 }
 

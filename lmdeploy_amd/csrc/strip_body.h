@@ -37,6 +37,7 @@ struct StripParams {
     int             rem;   // the first `rem` strips have base + 1
     int             epilogue;  // read by kernels whose epilogue is chosen at run time (EPI == kEpiRuntime)
     int             passes;    // strips per workgroup, one after the other (strip number = pass * workgroups + workgroup)
+    unsigned long long* clk = nullptr;  // measurement aid (clock_record_start / _stop); null in every ordinary launch
 };
 
 constexpr int kEpiRuntime = 3;  // template value: take the epilogue from StripParams

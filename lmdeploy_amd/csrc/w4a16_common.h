@@ -121,4 +121,26 @@ __device__ __forceinline__ void split_q(uint32_t q, half2_t& z1024, half2_t& z64
     s               = scale_is_normal(q) ? h[1] : (half_t)0.f;
 }
 
+// Measurement aid: the engine clock a kernel ran at.  One thread of a launch subtracts the core-clock counter and the
+// constant-rate counter from clk[0] and clk[1] when it starts and adds them when it ends (clk[2] counts launches), so
+// that nothing stays in a register in between; summed over launches, clk[0] / clk[1] x the constant rate is the
+// clock.  clk == nullptr (every ordinary launch) records nothing.
+__device__ __forceinline__ void clock_record_start(unsigned long long* clk, bool this_thread)
+{
+    if (clk != nullptr && this_thread) {
+        atomicAdd(clk, 0ull - (unsigned long long)clock64());
+        atomicAdd(clk + 1, 0ull - (unsigned long long)wall_clock64());
+        // (the kernels that follow wait for their loads by count: nothing else may be in flight)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+}
+__device__ __forceinline__ void clock_record_stop(unsigned long long* clk, bool this_thread)
+{
+    if (clk != nullptr && this_thread) {
+        atomicAdd(clk, (unsigned long long)clock64());
+        atomicAdd(clk + 1, (unsigned long long)wall_clock64());
+        atomicAdd(clk + 2, 1ull);
+    }
+}
+
 }  // namespace w4a16

@@ -21,6 +21,7 @@ struct GemmArgs {
     const uint16_t* R;   // fp16 residual [T, N] or null
     int             N, T, K;
     int             epilogue;
+    unsigned long long* clk = nullptr;  // measurement aid: where a strip kernel adds its cycle and tick counts (3 words)
 };
 
 // One dispatchable kernel configuration.
@@ -119,8 +120,10 @@ hipError_t launch_probe_read(const void* src, size_t bytes, void* sink, int cus,
 // the same with the GEMM kernels' load pipeline: `in_flight` (2, 4, 8, 16) loads of 16 bytes per lane kept in
 // flight by count, `wg_per_cu` (1, 2, 4) workgroups of eight waves per CU, hint 0 none / 1 nt / 2 sc0 sc1
 bool       probe_stream_config_ok(int wg_per_cu, int in_flight, int hint);
+// (clk: optional counters of clock_record_start / _stop)
+hipError_t launch_probe_mfma(void* sink, int cus, int waves_per_cu, int iters, unsigned long long* clk, hipStream_t st);
 hipError_t launch_probe_stream(const void* src, size_t bytes, void* sink, int cus, int wg_per_cu, int in_flight, int hint,
-                               hipStream_t st);
+                               hipStream_t st, unsigned long long* clk = nullptr);
 
 // decode (skinny) kernels
 bool       decode_feasible(const DecodeConfig& cf, int N, int T, int K);

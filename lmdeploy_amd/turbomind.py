@@ -215,6 +215,28 @@ class GemmS4F16:
         """Measurement aid: one persistent launch that crosses `iters` device-wide barriers and nothing else."""
         check(lib.w4a16_probe_barrier(self._h, iters, int(tree), _stream() if stream is None else stream))
 
+    def probe_mfma(self, waves_per_cu: int, iters: int, stream: Optional[int] = None) -> int:
+        """Measurement aid: nothing but matrix instructions, one workgroup of `waves_per_cu` waves per CU;
+        returns the flop the launch executes."""
+        check(lib.w4a16_probe_mfma(self._h, waves_per_cu, iters, _stream() if stream is None else stream))
+        return torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count * waves_per_cu * iters * 65536
+
+    def clock_begin(self, stream: Optional[int] = None) -> None:
+        """Measurement aid: from now on the decode strip kernels and the probes launched through this
+        operator record the engine cycles and constant-rate ticks they take (`clock_end` reads them)."""
+        check(lib.w4a16_probe_clock_begin(self._h, _stream() if stream is None else stream))
+
+    def clock_end(self, stream: Optional[int] = None) -> dict:
+        """Synchronises, stops the recording and returns {"MHz", "us_per_launch", "launches"} of the kernels
+        that recorded since `clock_begin` (zeros if none did)."""
+        c, t, n, r = ctypes.c_ulonglong(), ctypes.c_ulonglong(), ctypes.c_ulonglong(), ctypes.c_longlong()
+        check(lib.w4a16_probe_clock_end(self._h, ctypes.byref(c), ctypes.byref(t), ctypes.byref(n), ctypes.byref(r),
+                                        _stream() if stream is None else stream))
+        if not t.value or not n.value:
+            return {"MHz": 0.0, "us_per_launch": 0.0, "launches": int(n.value)}
+        return {"MHz": c.value / t.value * r.value / 1e6, "us_per_launch": t.value / n.value / r.value * 1e6,
+                "launches": int(n.value)}
+
     def pick(self, m: int, n: int, k: int) -> int:
         """The algo_id that `Run(..., algo_id=-1)` uses for this shape: the fastest one a previous
         `Measure` of exactly this shape found, else the heuristic's choice."""

@@ -659,6 +659,27 @@ def test_measure_reports_all_kernels(tm, gemm):
         gemm.pick(N + 8, T, K)
 
 
+def test_clock_recording_changes_no_result_and_reads_a_plausible_clock(tm):
+    """The measurement aid that records the engine clock inside the strip kernels: same outputs with and without it,
+    a clock between 1 and 3 GHz, one record per launch; and the MFMA probe runs and records too."""
+    g = tm.GemmS4F16()
+    K, N, T = 1024, 4096, 5
+    d = O.make_inputs(77, T, K, N)
+    A, Q = convert(tm, d, N, K)
+    plain = run(tm, g, d, A, Q, T, K, N, 0)
+    g.clock_begin()
+    rec = [run(tm, g, d, A, Q, T, K, N, 0) for _ in range(3)]
+    c = g.clock_end()
+    assert all(np.array_equal(r, plain) for r in rec)
+    assert c["launches"] == 3 and 1000 < c["MHz"] < 3000 and 0 < c["us_per_launch"] < 1000, c
+    again = run(tm, g, d, A, Q, T, K, N, 0)       # recording is off again
+    assert np.array_equal(again, plain) and g.clock_end()["launches"] == 3
+    g.clock_begin()
+    flop = g.probe_mfma(8, 1000)
+    c = g.clock_end()
+    assert flop > 0 and c["launches"] == 1 and 1000 < c["MHz"] < 3000, c
+
+
 def test_measured_choices_survive_in_a_file(tm, tmp_path):
     """w4a16_measure -> w4a16_save_tuning -> a fresh handle -> w4a16_load_tuning: the fresh handle then picks
     what was measured; a file written for another library version or CU count is refused and changes nothing."""

@@ -146,6 +146,12 @@ def test_static_and_sequence_argument_validation(L):
     assert lib.w4a16_probe_barrier(None, 10, 1, None) == L.EARG
     assert lib.w4a16_probe_stream(None, P, 1024, 1, 4, 1, None) == L.EARG
     assert lib.w4a16_probe_stream(FAKE, P, 1024, 3, 4, 1, None) == L.EARG and "wg_per_cu" in err(L)
+    assert lib.w4a16_probe_mfma(None, 8, 10, None) == L.EARG
+    assert lib.w4a16_probe_mfma(FAKE, 3, 10, None) == L.EARG and "waves_per_cu" in err(L)
+    assert lib.w4a16_probe_mfma(FAKE, 8, 0, None) == L.EARG and "iters" in err(L)
+    assert lib.w4a16_probe_clock_begin(None, None) == L.EARG
+    assert lib.w4a16_probe_clock_end(None, None, None, None, None, None) == L.EARG
+    assert lib.w4a16_probe_clock_end(FAKE, None, None, None, None, None) == L.EARG and "null output" in err(L)
 
 
 def test_deploy_entry_point_validation(L):
