@@ -191,7 +191,8 @@ int algo_pick(int N, int T, int K, const Scratch& lim)
     }
     // Decode.  Strips of column tiles over the whole of K, one per CU, were the fastest on every
     // Llama-7B/70B shape measured at 1..16 tokens; two narrower strips per CU are slightly ahead on
-    // very wide matrices while the activations are small.  Matrices with too few column tiles to
+    // very wide matrices while the activations are small (up to 4 tokens: 7B gate_up 11.5 against 12.0 us at
+    // one token, 13.2 against 12.4 at eight - a wide strip shares the sums of its activations among more tiles).  Matrices with too few column tiles to
     // give every CU a strip fall back to the column-block kernel, which can also split K across
     // workgroups.
     // Above 16 tokens every workgroup re-reads the weights once per 16-token block, and narrow
@@ -199,7 +200,7 @@ int algo_pick(int N, int T, int K, const Scratch& lim)
     if (N / 16 >= 128 && (T <= 16 || N / 16 >= 512)) {
         // (3 = one workgroup per CU taking several strips in turn: only feasible, and then measured 2 - 6 % ahead, for
         // matrices too wide for one strip per CU, such as the 57344 columns of Llama-2-70B's gate_up)
-        const int want = (N / 16 >= 1024 && T <= 8) ? 2 : 1;
+        const int want = (N / 16 >= 1024 && T <= 4) ? 2 : 1;
         for (int per_cu : {3, want, 1}) {
             for (int id = 0; id < algo_count(); ++id) {
                 const Algo& a = algo_at(id);
