@@ -37,7 +37,8 @@ int w4a16_probe_mfma(w4a16_handle* h, int waves_per_cu, int iters, void* stream)
  * it starts and when it ends and adds the differences up (launches captured into a graph in between keep
  * recording on every replay).  `end` synchronises the stream and returns the sums: cycles / ticks x
  * ticks_per_second is the clock those kernels ran at, ticks / launches their duration.  Ordinary launches
- * carry a null pointer and record nothing.  `begin` clears the counters on `stream`. */
+ * carry a null pointer and record nothing.  `begin` clears the counters on `stream` with a memset, so it is called
+ * outside stream capture; a handle records for one begin / end pair at a time. */
 int w4a16_probe_clock_begin(w4a16_handle* h, void* stream);
 int w4a16_probe_clock_end(w4a16_handle* h, unsigned long long* cycles, unsigned long long* ticks,
                           unsigned long long* launches, long long* ticks_per_second, void* stream);
