@@ -505,6 +505,11 @@ def main():
                 tf = fl / e0.elapsed_time(e1) / 1e9
                 mfma_loop["waves_per_cu_%d" % waves] = {"TFLOPs": round(tf, 1), "frac": round(tf / MFMA_PEAK_TFLOPS, 3),
                                                         "engine_clock_MHz": round(c["MHz"])}
+        # what one more kernel costs in a chain: 200 launches of a read of 256 KiB (warm) in one graph
+        tiny = torch.zeros(256 << 10, dtype=torch.uint8, device="cuda")
+        r = make_runner([[tiny] * 200], lambda w, st: [gemm.probe_stream(b, 1, 2, 1, stream=st) for b in w])
+        launch_floor_us = timed(r, 5, 1, 5) * 1e3 / (5 * 200)
+        del tiny, r
         # the engine clock inside a streaming read and inside the decode kernel of gate_up
         bufs = [torch.zeros(45 << 20, dtype=torch.uint8, device="cuda") for _ in range(max(3, int(args.cold_gib * 1024 / 45) + 1))]
         clocks = {"read_45MiB_wg1_inflight4_nt": kernel_clock(bufs, lambda w, st: [gemm.probe_stream(b, 1, 4, 1, stream=st) for b in w])}
@@ -513,6 +518,7 @@ def main():
             clocks["gate_up_T%d" % T] = kernel_clock([("gate_up", c, T) for c in range(len(weights["gate_up"]))])
         ceilings = dict(reads, device_wide_barrier=barrier, device_copy_512MiB_GBps=round(copy_gbs, 1),
                         mfma_loop=mfma_loop, engine_clock_in_kernel=clocks,
+                        kernel_period_floor_in_graph_us=round(launch_floor_us, 2),
                         dense_fp16_gemm_gate_up_T2048_TFLOPs=round(dense_tf, 1),
                         note="read_*: w4a16_probe_read (plain streaming read, one launch per buffer in a HIP graph, cold buffers) and, "
                              "under counted_loads_us, w4a16_probe_stream (the GEMM kernels' load pipeline: wgN = workgroups of eight "
@@ -521,7 +527,8 @@ def main():
                              "torch copy_ (bytes read + written); torch.matmul fp16 (hipBLASLt); mfma_loop: w4a16_probe_mfma, "
                              "8 launches of 40000 x 4 MFMAs per wave; engine_clock_in_kernel (and llama70b rows): core-clock "
                              "cycles over constant-rate ticks between the first and last instruction of one wave per launch "
-                             "(w4a16_probe_clock_begin / _end), kernel_us = those ticks per launch")
+                             "(w4a16_probe_clock_begin / _end), kernel_us = those ticks per launch; kernel_period_floor_in_graph_us: "
+                             "200 launches of a 256 KiB read in one graph, time per launch")
 
     # ---- Llama-2-70B layer shapes (BASELINE configs[3]) -----------------------------------------
     llama70b = None
