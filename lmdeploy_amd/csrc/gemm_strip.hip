@@ -3,10 +3,11 @@
 // The weight matrix is a grid of 1 KiB tiles (16 columns x one 128-row quantisation group).
 // The column tiles are dealt out as evenly as possible to B workgroups, B a multiple of the CU
 // count: workgroup b owns a strip of R or R-1 adjacent column tiles over the whole of K.  Its
-// eight waves deal the groups of K out round-robin; a wave walks its groups and, per group,
-// loads the strip's R tiles (R KiB contiguous in the group-major tile layout) and its own
-// activations of that group straight into registers - no cooperative staging, no barrier and no
-// other wave involved until the end, when the eight partial strips are added in LDS in slice order.
+// eight waves (sixteen for one-tile strips at up to four tokens) deal the groups of K out
+// round-robin; a wave walks its groups and, per group, loads the strip's R tiles (R KiB contiguous
+// in the group-major tile layout) and its own activations of that group straight into registers -
+// no cooperative staging, no barrier and no other wave involved until the end, when the partial
+// strips are added in LDS in slice order.
 //
 // Why this shape: (a) every CU gets the same number of tiles to within one strip column, which
 // the column-block decomposition could not offer for matrices like 4096 x 22016 (1376 column
@@ -55,6 +56,29 @@ __global__ void __launch_bounds__(64 * kWaves) strip_kernel(const StripParams p)
         if (!done) strip_body<RMAX, TP, EPI>(p, col0, smem);
     }
     clock_record_stop(p.clk, blockIdx.x == gridDim.x / 2 && blockIdx.y == 0 && threadIdx.x == 0);
+}
+
+// One-tile strips at up to four tokens: sixteen waves instead of eight, so that a wave walks half as many groups
+// one after the other (7B down at one token: 8.6 -> 7.6 us, o: 4.65 -> 4.5; two-tile strips and eight tokens and
+// more are better off with eight waves).
+constexpr int kWavesNarrow = 16;
+template<int EPI>
+__global__ void __launch_bounds__(64 * kWavesNarrow) strip_kernel_narrow(const StripParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) u32x4_t smem[];
+    clock_record_start(p.clk, blockIdx.x == gridDim.x / 2 && threadIdx.x == 0);
+    strip_body<1, 4, EPI, false, kWavesNarrow>(p, (int)blockIdx.x, smem);
+    clock_record_stop(p.clk, blockIdx.x == gridDim.x / 2 && threadIdx.x == 0);
+}
+
+hipError_t launch_narrow(const StripParams& p, dim3 grid, size_t lds, int epilogue, hipStream_t st)
+{
+    const dim3 block(64 * kWavesNarrow);
+    switch (epilogue) {
+        case kEpiGemm: return launch_kernel(strip_kernel_narrow<kEpiGemm>, grid, block, lds, st, p);
+        case kEpiSilu: return launch_kernel(strip_kernel_narrow<kEpiSilu>, grid, block, lds, st, p);
+        default: return launch_kernel(strip_kernel_narrow<kEpiAdd>, grid, block, lds, st, p);
+    }
 }
 
 // The same kernel for group sizes 64 and 32 (NQ = 2, 4 quantisation groups per 128-row tile): 16 token rows per
@@ -210,6 +234,8 @@ hipError_t strip_launch(int per_cu, int block_t, const GemmArgs& a, hipStream_t 
     const dim3   grid(pl.strips, (a.T + block_t - 1) / block_t);
     // per wave: the sums of its strip, over its activation patch(es) - two for 32 tokens, which arrive straight from memory
     const size_t lds = (size_t)kWaves * std::max(pl.rmax * h * 1024, tp * 256 * (tp >= kDmaTokens ? 2 : 1));
+    if (tp == 4 && pl.rmax == 1 && pl.passes == 1 && a.K / kGroup >= 2 * kWavesNarrow)
+        return launch_narrow(p, grid, (size_t)kWavesNarrow * 1024, a.epilogue, st);
     switch (pl.rmax) {
         case 1: return launch_r<1>(tp, p, grid, lds, a.epilogue, st);
         case 2: return launch_r<2>(tp, p, grid, lds, a.epilogue, st);
