@@ -36,7 +36,8 @@ namespace {
 using namespace strip;
 
 // RMAX = width of the wide strips (base + 1 when the column tiles do not divide evenly).
-template<int RMAX, int TP, int EPI>
+// D = groups in flight per wave (2, or 1 for wide strips: see strip_launch).
+template<int RMAX, int TP, int EPI, int D = 2>
 __global__ void __launch_bounds__(64 * kWaves) strip_kernel(const StripParams p)
 {
     extern __shared__ __attribute__((aligned(16))) u32x4_t smem[];  // activation patches [8][1 or 2][TP][16], then sums [8][R][H][64]
@@ -49,11 +50,11 @@ __global__ void __launch_bounds__(64 * kWaves) strip_kernel(const StripParams p)
         bool done = false;
         if constexpr (RMAX > 1) {
             if (!wide && p.base == RMAX - 1) {
-                strip_body<RMAX - 1, TP, EPI>(p, col0, smem);
+                strip_body<RMAX - 1, TP, EPI, false, kWaves, NoWait, 1, D>(p, col0, smem);
                 done = true;
             }
         }
-        if (!done) strip_body<RMAX, TP, EPI>(p, col0, smem);
+        if (!done) strip_body<RMAX, TP, EPI, false, kWaves, NoWait, 1, D>(p, col0, smem);
     }
     clock_record_stop(p.clk, blockIdx.x == gridDim.x / 2 && blockIdx.y == 0 && threadIdx.x == 0);
 }
@@ -117,13 +118,14 @@ hipError_t launch_q(int rmax, const StripParams& p, dim3 grid, size_t lds, hipSt
     }
 }
 
-template<int RMAX, int TP>
+constexpr int kMinRShallow = 3;  // narrowest strip that exists with one group in flight per wave
+template<int RMAX, int TP, int D = 2>
 hipError_t launch_rt(const StripParams& p, dim3 grid, size_t lds, int epilogue, hipStream_t st)
 {
     const dim3 block(64 * kWaves);
 #define W4A16_LAUNCH(EPI)                                                                                              \
     do {                                                                                                               \
-        auto kfn = strip_kernel<RMAX, TP, EPI>;                                                                        \
+        auto kfn = strip_kernel<RMAX, TP, EPI, D>;                                                                     \
         if constexpr (TP == 32) { /* up to 128 KiB of LDS: above the default limit */                                  \
             static std::atomic<uint64_t> raised{0};                                                                    \
             const hipError_t e = raise_lds_limit(reinterpret_cast<const void*>(kfn), 8 * kMaxR32 * 2 * 1024, raised);  \
@@ -140,8 +142,18 @@ hipError_t launch_rt(const StripParams& p, dim3 grid, size_t lds, int epilogue, 
 }
 
 template<int RMAX>
-hipError_t launch_r(int tp, const StripParams& p, dim3 grid, size_t lds, int epilogue, hipStream_t st)
+hipError_t launch_r(int tp, int depth, const StripParams& p, dim3 grid, size_t lds, int epilogue, hipStream_t st)
 {
+    if constexpr (RMAX >= kMinRShallow) {
+        if (depth == 1) {
+            switch (tp) {
+                case 4: return launch_rt<RMAX, 4, 1>(p, grid, lds, epilogue, st);
+                case 8: return launch_rt<RMAX, 8, 1>(p, grid, lds, epilogue, st);
+                case 16: return launch_rt<RMAX, 16, 1>(p, grid, lds, epilogue, st);
+                default: break;  // 32 tokens per workgroup: two groups in flight only
+            }
+        }
+    }
     switch (tp) {
         case 4: return launch_rt<RMAX, 4>(p, grid, lds, epilogue, st);
         case 8: return launch_rt<RMAX, 8>(p, grid, lds, epilogue, st);
@@ -236,15 +248,21 @@ hipError_t strip_launch(int per_cu, int block_t, const GemmArgs& a, hipStream_t 
     const size_t lds = (size_t)kWaves * std::max(pl.rmax * h * 1024, tp * 256 * (tp >= kDmaTokens ? 2 : 1));
     if (tp == 4 && pl.rmax == 1 && pl.passes == 1 && a.K / kGroup >= 2 * kWavesNarrow)
         return launch_narrow(p, grid, (size_t)kWavesNarrow * 1024, a.epilogue, st);
+    // Two groups per wave in flight are waves x 2 x R KiB per CU.  The memory system streams fastest with 32 - 64 KiB
+    // requested per CU (more is slower); beyond that every wave keeps one group in flight instead: 7B gate_up
+    // 12.9 -> 12.2 us at 16 tokens (strips of 6) and 11.4 -> 11.2 at one (two workgroups of 3 per CU), 70B gate_up
+    // 44.8 -> 43.5; narrower strips lose (qkv, strips of 3: 7.4 -> 8.0).
+    const int waves_per_cu = kWaves * ((pl.strips + device_cus() - 1) / device_cus());
+    const int depth        = waves_per_cu * 2 * pl.rmax > 64 ? 1 : 2;
     switch (pl.rmax) {
-        case 1: return launch_r<1>(tp, p, grid, lds, a.epilogue, st);
-        case 2: return launch_r<2>(tp, p, grid, lds, a.epilogue, st);
-        case 3: return launch_r<3>(tp, p, grid, lds, a.epilogue, st);
-        case 4: return launch_r<4>(tp, p, grid, lds, a.epilogue, st);
-        case 5: return launch_r<5>(tp, p, grid, lds, a.epilogue, st);
-        case 6: return launch_r<6>(tp, p, grid, lds, a.epilogue, st);
-        case 7: return launch_r<7>(tp, p, grid, lds, a.epilogue, st);
-        default: return launch_r<8>(tp, p, grid, lds, a.epilogue, st);
+        case 1: return launch_r<1>(tp, depth, p, grid, lds, a.epilogue, st);
+        case 2: return launch_r<2>(tp, depth, p, grid, lds, a.epilogue, st);
+        case 3: return launch_r<3>(tp, depth, p, grid, lds, a.epilogue, st);
+        case 4: return launch_r<4>(tp, depth, p, grid, lds, a.epilogue, st);
+        case 5: return launch_r<5>(tp, depth, p, grid, lds, a.epilogue, st);
+        case 6: return launch_r<6>(tp, depth, p, grid, lds, a.epilogue, st);
+        case 7: return launch_r<7>(tp, depth, p, grid, lds, a.epilogue, st);
+        default: return launch_r<8>(tp, depth, p, grid, lds, a.epilogue, st);
     }
 }
 

@@ -143,7 +143,9 @@ struct NoWait {
 // NQ: quantisation groups per 128-row weight tile (group sizes 128, 64, 32 = NQ 1, 2, 4).  The weight layout does
 // not depend on it; Q then has NQ rows per tile row, and every 128 / NQ rows of a tile have their own scale and
 // zero point: NQ shorter MFMA chains per tile, each scaled into the accumulator by itself.
-template<int R, int TP, int EPI, bool SEQ = false, int NW = kWaves, typename Ready = NoWait, int NQ = 1>
+// DD: groups in flight per wave.  Two, unless the strip is so wide that two groups of it from every wave of the CU
+// are more than the memory system takes at once (the launcher decides); then one.
+template<int R, int TP, int EPI, bool SEQ = false, int NW = kWaves, typename Ready = NoWait, int NQ = 1, int DD = 2>
 __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4_t* smem, Ready&& inputs_ready = Ready{})
 {
     const int tid  = threadIdx.x;
@@ -178,7 +180,8 @@ __device__ __forceinline__ void strip_body(const StripParams& p, int col0, u32x4
     // With 32 tokens the rows go from global memory straight into the patch instead (no registers, no
     // LDS write), one patch per group in flight; the swizzle is then applied on the way in: the lane
     // that lands at position p of row r fetches chunk p ^ r.
-    constexpr int  D    = 2;  // groups in flight per wave
+    constexpr int  D    = DD;  // groups in flight per wave
+    static_assert(D == 2 || (D == 1 && !SEQ), "one or two groups in flight");
     constexpr bool XDMA = TP >= kDmaTokens && !SEQ;
     constexpr int  NX   = TP / 4;
     constexpr int  NXR  = XDMA ? 0 : NX;  // activation loads that land in registers
