@@ -150,7 +150,9 @@ hipError_t launch_r(int tp, int depth, const StripParams& p, dim3 grid, size_t l
                 case 4: return launch_rt<RMAX, 4, 1>(p, grid, lds, epilogue, st);
                 case 8: return launch_rt<RMAX, 8, 1>(p, grid, lds, epilogue, st);
                 case 16: return launch_rt<RMAX, 16, 1>(p, grid, lds, epilogue, st);
-                default: break;  // 32 tokens per workgroup: two groups in flight only
+                default:
+                    if constexpr (RMAX <= kMaxR32) return launch_rt<RMAX, 32, 1>(p, grid, lds, epilogue, st);
+                    break;
             }
         }
     }
@@ -250,8 +252,8 @@ hipError_t strip_launch(int per_cu, int block_t, const GemmArgs& a, hipStream_t 
         return launch_narrow(p, grid, (size_t)kWavesNarrow * 1024, a.epilogue, st);
     // Two groups per wave in flight are waves x 2 x R KiB per CU.  The memory system streams fastest with 32 - 64 KiB
     // requested per CU (more is slower); beyond that every wave keeps one group in flight instead: 7B gate_up
-    // 12.9 -> 12.2 us at 16 tokens (strips of 6) and 11.4 -> 11.2 at one (two workgroups of 3 per CU), 70B gate_up
-    // 44.8 -> 43.5; narrower strips lose (qkv, strips of 3: 7.4 -> 8.0).
+    // 12.9 -> 12.2 us at 16 tokens (strips of 6), 16.9 -> 15.7 at 32, and 11.4 -> 11.2 at one (two workgroups of 3 per
+    // CU), 70B gate_up 44.8 -> 43.5; narrower strips lose (qkv, strips of 3: 7.4 -> 8.0).
     const int waves_per_cu = kWaves * ((pl.strips + device_cus() - 1) / device_cus());
     const int depth        = waves_per_cu * 2 * pl.rmax > 64 ? 1 : 2;
     switch (pl.rmax) {
