@@ -659,6 +659,21 @@ def test_measure_reports_all_kernels(tm, gemm):
         gemm.pick(N + 8, T, K)
 
 
+@pytest.mark.parametrize("K,N,tokens", [(4224, 64, (1, 3, 4)), (4224, 4096, (1, 2, 4)), (4224, 22016, (1, 4, 8, 16)),
+                                         (11008, 4096, (1, 4))])
+def test_narrow_and_wide_strip_variants(tm, gemm, K, N, tokens):
+    """The strip kernel's variants that the launcher picks by strip width: sixteen waves for one-tile strips at up to
+    four tokens (64 and 4096 columns), one group in flight per wave for wide strips (22016 columns); 33 groups of K
+    do not divide by the waves of either."""
+    d0 = O.make_inputs(900 + N, max(tokens), K, N, residual=True)
+    A, Q = convert(tm, d0, N, K)
+    for T in tokens:
+        d = dict(d0, X=d0["X"][:T], R=d0["R"][:T])
+        for kind in (0, 1, 2):
+            want = O.gemm_s4_f16(d["X"], d["qweight"], d["qzeros"], d["scales"], 128, kind, d["R"])
+            assert_close(run(tm, gemm, d, A, Q, T, K, N, kind), want, (K, N, T, kind))
+
+
 def test_clock_recording_changes_no_result_and_reads_a_plausible_clock(tm):
     """The measurement aid that records the engine clock inside the strip kernels: same outputs with and without it,
     a clock between 1 and 3 GHz, one record per launch; and the MFMA probe runs and records too."""
