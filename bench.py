@@ -108,6 +108,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=24)
     ap.add_argument("--repeats", type=int, default=9,
                     help="the timed region of --steps steps is measured this many times in a row; the median is reported")
+    ap.add_argument("--steps-per-graph", type=int, default=4,
+                    help="steps captured into one HIP graph (must divide --steps); a decode step of a whole model is one "
+                         "graph of hundreds of launches, so what one graph launch costs is spread thinner there")
     ap.add_argument("--copies", type=int, default=12,
                     help="distinct sets of 16 weight matrices (one per GEMM of a step) the steps rotate through")
     ap.add_argument("--cold-gib", type=float, default=1.25,
@@ -131,6 +134,9 @@ def main():
                          "rate once a second, so that the engine clock under that load can be read beside it "
                          "(`rocm-smi --showclocks`)")
     args = ap.parse_args()
+    if args.steps_per_graph < 1 or args.steps % args.steps_per_graph:
+        print("bench.py: --steps-per-graph must divide --steps", file=sys.stderr)
+        sys.exit(2)
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
@@ -292,11 +298,14 @@ def main():
 
     # ---- headline: the decode layer set; every GEMM of a step has its own weight copy ----------
     step_bytes = sum(algorithmic_bytes(T, K, N, epi) for T in DECODE_T for _, K, N, epi in LAYER_7B)
-    runner = make_runner([[(name, len(DECODE_T) * c + ti, T) for ti, T in enumerate(DECODE_T) for name, _, _, _ in LAYER_7B]
-                          for c in range(n_sets)])
+    def set_work(c):
+        return [(name, len(DECODE_T) * c + ti, T) for ti, T in enumerate(DECODE_T) for name, _, _, _ in LAYER_7B]
+
+    S = args.steps_per_graph
+    runner = make_runner([sum((set_work((g * S + j) % n_sets) for j in range(S)), []) for g in range(n_sets)])
     # One timed region of `steps` steps lasts a few milliseconds and cannot resolve a 3 % change; the region is
     # therefore timed `--repeats` times in a row and the median region is the one reported.
-    regions = sorted(timed_all(runner, args.steps, args.warmup, args.repeats))
+    regions = sorted(timed_all(runner, args.steps // S, max(1, args.warmup // S), args.repeats))
     ms = regions[len(regions) // 2]
     ms_per_step = ms / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
@@ -621,7 +630,7 @@ def main():
         "config": {"workload": "Llama-2-7B decode layer set (qkv 4096x12288, o 4096x4096, gate_up 4096x22016 +SiLU, "
                                "down 11008x4096 +residual) at T in {1,4,8,16}, group 128: 16 GEMMs per step, each on its own "
                                "weight copy, %d rotating sets of 16" % n_sets,
-                   "launch": "eager" if args.eager else "hipgraph replay of one step",
+                   "launch": "eager" if args.eager else "hipgraph replays, %d steps (%d launches) per graph" % (S, 16 * S),
                    "bytes_per_step": step_bytes},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "roofline": roofline, "roofline_worst_decode_kernel": roofline_worst, "cpu_baseline": cpu,
