@@ -108,8 +108,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=24)
     ap.add_argument("--repeats", type=int, default=9,
                     help="the timed region of --steps steps is measured this many times in a row; the median is reported")
-    ap.add_argument("--steps-per-graph", type=int, default=4,
-                    help="steps captured into one HIP graph (must divide --steps); a decode step of a whole model is one "
+    ap.add_argument("--steps-per-graph", type=int, default=0,
+                    help="steps captured into one HIP graph (must divide --steps; 0 = 4, or else 5, 3, 2 or 1, whichever "
+                         "divides --steps first); a decode step of a whole model is one "
                          "graph of hundreds of launches, so what one graph launch costs is spread thinner there")
     ap.add_argument("--copies", type=int, default=12,
                     help="distinct sets of 16 weight matrices (one per GEMM of a step) the steps rotate through")
@@ -134,7 +135,9 @@ def main():
                          "rate once a second, so that the engine clock under that load can be read beside it "
                          "(`rocm-smi --showclocks`)")
     args = ap.parse_args()
-    if args.steps_per_graph < 1 or args.steps % args.steps_per_graph:
+    if args.steps_per_graph == 0:
+        args.steps_per_graph = next(s for s in (4, 5, 3, 2, 1) if args.steps % s == 0)
+    if args.steps < 1 or args.steps_per_graph < 1 or args.steps % args.steps_per_graph:
         print("bench.py: --steps-per-graph must divide --steps", file=sys.stderr)
         sys.exit(2)
     if args.gpus != 1:
