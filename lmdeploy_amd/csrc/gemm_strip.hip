@@ -3,7 +3,7 @@
 // The weight matrix is a grid of 1 KiB tiles (16 columns x one 128-row quantisation group).
 // The column tiles are dealt out as evenly as possible to B workgroups, B a multiple of the CU
 // count: workgroup b owns a strip of R or R-1 adjacent column tiles over the whole of K.  Its
-// eight waves (sixteen for one-tile strips at up to four tokens) deal the groups of K out
+// eight waves (sixteen for one-tile strips at up to eight tokens) deal the groups of K out
 // round-robin; a wave walks its groups and, per group, loads the strip's R tiles (R KiB contiguous
 // in the group-major tile layout) and its own activations of that group straight into registers -
 // no cooperative staging, no barrier and no other wave involved until the end, when the partial
@@ -59,26 +59,30 @@ __global__ void __launch_bounds__(64 * kWaves) strip_kernel(const StripParams p)
     clock_record_stop(p.clk, blockIdx.x == gridDim.x / 2 && blockIdx.y == 0 && threadIdx.x == 0);
 }
 
-// One-tile strips at up to four tokens: sixteen waves instead of eight, so that a wave walks half as many groups
-// one after the other (7B down at one token: 8.6 -> 7.6 us, o: 4.65 -> 4.5; two-tile strips and eight tokens and
-// more are better off with eight waves).
+// One-tile strips at up to eight tokens: sixteen waves instead of eight, so that a wave walks half as many groups
+// one after the other and the CU has 32 KiB of weights requested instead of 16 (7B down at one token: 8.6 -> 7.6 us,
+// o: 4.65 -> 4.5).  At five to eight tokens the activation rows double what a stage holds, and each wave keeps one
+// group in flight instead of two (down at eight tokens 9.7 -> 9.1 us, o 5.0 -> 4.85); at sixteen tokens, and for
+// two-tile strips, eight waves are ahead.
 constexpr int kWavesNarrow = 16;
-template<int EPI>
+template<int TP, int EPI, int D>
 __global__ void __launch_bounds__(64 * kWavesNarrow) strip_kernel_narrow(const StripParams p)
 {
     extern __shared__ __attribute__((aligned(16))) u32x4_t smem[];
     clock_record_start(p.clk, blockIdx.x == gridDim.x / 2 && threadIdx.x == 0);
-    strip_body<1, 4, EPI, false, kWavesNarrow>(p, (int)blockIdx.x, smem);
+    strip_body<1, TP, EPI, false, kWavesNarrow, NoWait, 1, D>(p, (int)blockIdx.x, smem);
     clock_record_stop(p.clk, blockIdx.x == gridDim.x / 2 && threadIdx.x == 0);
 }
 
-hipError_t launch_narrow(const StripParams& p, dim3 grid, size_t lds, int epilogue, hipStream_t st)
+template<int TP, int D>
+hipError_t launch_narrow(const StripParams& p, dim3 grid, int epilogue, hipStream_t st)
 {
-    const dim3 block(64 * kWavesNarrow);
+    const dim3   block(64 * kWavesNarrow);
+    const size_t lds = (size_t)kWavesNarrow * std::max(1024, TP * 256);
     switch (epilogue) {
-        case kEpiGemm: return launch_kernel(strip_kernel_narrow<kEpiGemm>, grid, block, lds, st, p);
-        case kEpiSilu: return launch_kernel(strip_kernel_narrow<kEpiSilu>, grid, block, lds, st, p);
-        default: return launch_kernel(strip_kernel_narrow<kEpiAdd>, grid, block, lds, st, p);
+        case kEpiGemm: return launch_kernel(strip_kernel_narrow<TP, kEpiGemm, D>, grid, block, lds, st, p);
+        case kEpiSilu: return launch_kernel(strip_kernel_narrow<TP, kEpiSilu, D>, grid, block, lds, st, p);
+        default: return launch_kernel(strip_kernel_narrow<TP, kEpiAdd, D>, grid, block, lds, st, p);
     }
 }
 
@@ -248,8 +252,8 @@ hipError_t strip_launch(int per_cu, int block_t, const GemmArgs& a, hipStream_t 
     const dim3   grid(pl.strips, (a.T + block_t - 1) / block_t);
     // per wave: the sums of its strip, over its activation patch(es) - two for 32 tokens, which arrive straight from memory
     const size_t lds = (size_t)kWaves * std::max(pl.rmax * h * 1024, tp * 256 * (tp >= kDmaTokens ? 2 : 1));
-    if (tp == 4 && pl.rmax == 1 && pl.passes == 1 && a.K / kGroup >= 2 * kWavesNarrow)
-        return launch_narrow(p, grid, (size_t)kWavesNarrow * 1024, a.epilogue, st);
+    if (tp <= 8 && pl.rmax == 1 && pl.passes == 1 && a.K / kGroup >= 2 * kWavesNarrow)
+        return tp == 4 ? launch_narrow<4, 2>(p, grid, a.epilogue, st) : launch_narrow<8, 1>(p, grid, a.epilogue, st);
     // Two groups per wave in flight are waves x 2 x R KiB per CU.  The memory system streams fastest with 32 - 64 KiB
     // requested per CU (more is slower); beyond that every wave keeps one group in flight instead: 7B gate_up
     // 12.9 -> 12.2 us at 16 tokens (strips of 6), 16.9 -> 15.7 at 32, and 11.4 -> 11.2 at one (two workgroups of 3 per
