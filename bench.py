@@ -346,6 +346,8 @@ def main():
                 by = algorithmic_bytes(T, K, N, epi)
                 per_shape.append({"shape": name, "T": T, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
                                   "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 3)})
+                if T in (1, 16):   # the engine clock inside the kernel and the life of one of its workgroups
+                    per_shape[-1]["engine_clock"] = kernel_clock([(name, c, T) for c in range(len(weights[name]))])
 
     # ---- batched decode / short prompts: 32 .. 256 tokens (not part of `value`) ----------------
     batched = []
